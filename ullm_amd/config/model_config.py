@@ -10,7 +10,7 @@ from __future__ import annotations
 import json
 import os
 from dataclasses import asdict, dataclass, fields
-from typing import Any, Mapping
+from typing import Any, Mapping, Optional
 
 
 class ConfigError(ValueError):
@@ -209,3 +209,89 @@ def read_config_json(model_dir: str) -> dict:
 
 def config_field_names(cls) -> list:
     return [f.name for f in fields(cls)]
+
+
+@dataclass(frozen=True)
+class PamopelLayer:
+    """One layer of a Pamopel config.json: ``type`` names the mixer, ``mixer`` holds its sizes and constants as
+    (key, value) pairs, ``mlp`` those of the feed-forward or None for a layer without one."""
+    type: str
+    mixer: tuple
+    mlp: Optional[tuple]
+
+    def mixer_dict(self) -> dict:
+        return dict(self.mixer)
+
+    def mlp_dict(self) -> Optional[dict]:
+        return None if self.mlp is None else dict(self.mlp)
+
+
+_PAMOPEL_MIXER_KEYS = {
+    "attention": (("heads", int), ("kv_heads", int), ("dim", int), ("vdim", int), ("scale", float), ("bias_max", int)),
+    "mamba2": (("heads", int), ("vdim", int), ("state", int), ("groups", int), ("conv", int), ("norm_groups", int)),
+}
+
+
+@dataclass(frozen=True)
+class PamopelConfig:
+    """Keys of a Pamopel config.json: a stack whose layers are listed one by one (attention with a learned
+    bias by distance and a gate per head, possibly reading another layer's keys and values; or a Mamba-2
+    mixer), layer norms on both sides of every sublayer, and an embedding that adds a hashed bigram row and
+    a sinusoidal position row to the token's."""
+    architecture: str
+    vocab_size: int
+    hidden_size: int
+    layers: tuple                   # of PamopelLayer
+    norm_eps: float
+    residual_mult: float
+    logit_scale: float
+    embedding_scale: float
+    bigram_buckets: int             # 0: no bigram table
+    bigram_mul_prev: int
+    bigram_mul_cur: int
+
+    @classmethod
+    def from_dict(cls, d: Mapping[str, Any]) -> "PamopelConfig":
+        emb = d.get("embedding") or {}
+        if not isinstance(emb, Mapping):
+            raise ConfigError("config.json: key 'embedding' must be an object")
+        big = emb.get("bigram") or {}
+        norm = d.get("norm") or {}
+        raw_layers = d.get("layers")
+        if not isinstance(raw_layers, (list, tuple)) or not raw_layers:
+            raise ConfigError("config.json: key 'layers' must be a non-empty list")
+        layers = []
+        for i, L in enumerate(raw_layers):
+            kind = _take(L, "type", str)
+            if kind not in _PAMOPEL_MIXER_KEYS:
+                raise ConfigError(f"config.json: layer {i} has type {kind!r}; known: {sorted(_PAMOPEL_MIXER_KEYS)}")
+            m = L.get("mixer")
+            if not isinstance(m, Mapping):
+                raise ConfigError(f"config.json: layer {i} has no 'mixer' object")
+            try:
+                mixer = [(key, _take(m, key, typ)) for key, typ in _PAMOPEL_MIXER_KEYS[kind]]
+                if kind == "attention" and m.get("kv_from") is not None:
+                    src = _take(m, "kv_from", int)
+                    if not 0 <= src < i or raw_layers[src].get("type") != "attention" \
+                            or (raw_layers[src].get("mixer") or {}).get("kv_from") is not None:
+                        raise ConfigError(f"'kv_from': {src} must name an earlier attention layer with keys of its own")
+                    mixer.append(("kv_from", src))
+                mlp = L.get("mlp")
+                if mlp is not None:
+                    if not isinstance(mlp, Mapping) or _take(mlp, "kind", str) != "dense":
+                        raise ConfigError("'mlp' must be null or an object of kind 'dense'")
+                    mlp = (("kind", "dense"), ("ff", _take(mlp, "ff", int)))
+            except ConfigError as e:
+                raise ConfigError(f"{e} (layer {i})") from None
+            layers.append(PamopelLayer(kind, tuple(mixer), mlp))
+        return cls(
+            architecture=_take(d, "architecture", str, "Pamopel"),
+            vocab_size=_take(d, "vocab", int), hidden_size=_take(d, "width", int), layers=tuple(layers),
+            norm_eps=_take(norm, "eps", float), residual_mult=_take(d, "residual_mult", float, 1.0),
+            logit_scale=_take(d, "logit_scale", float, 1.0), embedding_scale=_take(emb, "scale", float, 1.0),
+            bigram_buckets=_take(big, "buckets", int, 0), bigram_mul_prev=_take(big, "mul_prev", int, 0),
+            bigram_mul_cur=_take(big, "mul_cur", int, 0))
+
+    @property
+    def num_hidden_layers(self) -> int:
+        return len(self.layers)

@@ -2,7 +2,9 @@
 // groups, any page size, any mix of prompt portions and single decoded tokens, optional window.
 // One block per (token, query head); keys are visited in tiles of the block size in a fixed order
 // that depends only on the token's own position, so the result for a token is the same however
-// the batch was cut.  Scores, running maximum, sum and output are 32-bit.
+// the batch was cut.  Scores, running maximum, sum and output are 32-bit.  Optionally a bias by
+// distance is added to every score: bias[head, min(query position - key position, bias_rows - 1)]
+// (float32 [nq, bias_rows]); the scale does not multiply it.
 // Pools: keys [page, kv_head, row, head_dim]; values [page, kv_head, head_dim, row].
 //
 // Semantics as the reference asks of its attention library (ullm/layers/attention.py:76-104,
@@ -19,7 +21,8 @@ paged_attention_generic_kernel(const T* __restrict__ q, int q_stride, T* __restr
                                const T* __restrict__ k_pool, const T* __restrict__ v_pool,
                                const int* __restrict__ positions, const int* __restrict__ token_entry,
                                const int* __restrict__ block_table, int bt_stride, int page_size,
-                               int nq, int nkv, int hd, float scale, int window) {
+                               int nq, int nkv, int hd, float scale, int window,
+                               const float* __restrict__ bias, int bias_rows) {
   __shared__ float q_s[ATT_MAX_HD];
   __shared__ float p_s[ATT_THREADS];
   __shared__ long long row_s[ATT_THREADS];
@@ -51,6 +54,8 @@ paged_attention_generic_kernel(const T* __restrict__ q, int q_stride, T* __restr
         const T* kp = k_pool + row * hd;
         float d = 0.f;
         for (int i = 0; i < hd; ++i) d += q_s[i] * ld_f32(kp + i);
+        // a learned bias by distance: one row of the table per head, the last entry for every greater distance
+        if (bias) d += bias[(size_t)h * bias_rows + (pos - j < bias_rows ? pos - j : bias_rows - 1)];
         s = d;
       }
     }
@@ -93,14 +98,16 @@ paged_attention_generic_kernel(const T* __restrict__ q, int q_stride, T* __restr
 extern "C" int ullm_paged_attention_generic(
     const void* q, int q_stride, void* out, int out_stride, const void* k_pool, const void* v_pool,
     const int* positions, const int* token_entry, const int* block_table, int bt_stride, int page_size,
-    int T_, int nq, int nkv, int hd, float scale, int window, int dtype, hipStream_t stream) {
+    int T_, int nq, int nkv, int hd, float scale, int window, const float* bias, int bias_rows, int dtype,
+    hipStream_t stream) {
   if (T_ <= 0) return 0;
+  if (bias && bias_rows <= 0) return ULLM_ERR_SHAPE;
   if (hd <= 0 || hd > ATT_MAX_HD || nq <= 0 || nkv <= 0 || nq % nkv != 0 || page_size <= 0 || window < 0)
     return ULLM_ERR_SHAPE;
   dim3 grid(T_, nq), block(ATT_THREADS);
 #define GO(TT) hipLaunchKernelGGL(paged_attention_generic_kernel<TT>, grid, block, 0, stream, \
     (const TT*)q, q_stride, (TT*)out, out_stride, (const TT*)k_pool, (const TT*)v_pool, positions, \
-    token_entry, block_table, bt_stride, page_size, nq, nkv, hd, scale, window)
+    token_entry, block_table, bt_stride, page_size, nq, nkv, hd, scale, window, bias, bias_rows)
   if (dtype == ULLM_F32) GO(float);
   else if (dtype == ULLM_BF16) GO(bf16_t);
   else return ULLM_ERR_DTYPE;

@@ -777,3 +777,265 @@ extern "C" int ullm_qk_norm_rope_write(
 #undef GO
   ULLM_LAUNCH_CHECK();
 }
+
+// ------------------------------------------------------------------ x *= s
+__global__ void scale_kernel(float* __restrict__ x, int cols, int ld, float s) {
+  float* row = x + (size_t)blockIdx.y * ld;
+  for (int c = blockIdx.x * blockDim.x + threadIdx.x; c < cols; c += gridDim.x * blockDim.x) row[c] *= s;
+}
+
+extern "C" int ullm_scale(float* x, int rows, int cols, int ld, float s, hipStream_t stream) {
+  if (rows <= 0 || cols <= 0) return 0;
+  if (ld < cols || rows > 65535) return ULLM_ERR_SHAPE;
+  int bx = (cols + 255) / 256;
+  if (bx > 64) bx = 64;
+  hipLaunchKernelGGL(scale_kernel, dim3(bx, rows), dim3(256), 0, stream, x, cols, ld, s);
+  ULLM_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------------------------ embedding as a sum of tables
+// stream[t, :] = scale * token_table[ids[t], :]
+//              + pair_table[row(t), :]              (if pair_table)
+//              + position_table[positions[t], :]    (if position_table; float32)
+// row(t) = pair_rows for a request's first token (the table's last row), else
+// (previous id * mul_prev + ids[t] * mul_cur) mod pair_rows.  The previous id of an entry's first token is
+// what the step before left in last_id[slot of the entry]; the block of that token reads it and then,
+// behind a barrier, leaves the entry's last id there for the next step.
+template <typename T>
+__global__ void __launch_bounds__(256)
+embedding_sum_kernel(const int* __restrict__ ids, const T* __restrict__ token_table, float scale,
+                     const T* __restrict__ pair_table, long long pair_rows, long long mul_prev, long long mul_cur,
+                     const float* __restrict__ position_table, int position_rows,
+                     const int* __restrict__ positions, const int* __restrict__ token_entry,
+                     const int* __restrict__ q_start, const int* __restrict__ entry_slot,
+                     int* __restrict__ last_id, float* __restrict__ stream, int H, int V) {
+  const int t = blockIdx.x;
+  const int b = token_entry[t];
+  const int first = q_start[b];
+  const int pos = positions[t];
+  int id = ids[t];
+  const bool known = id >= 0 && id < V;
+  if (!known) id = 0;
+  long long pair = -1;
+  if (pair_table) {
+    if (pos == 0) {
+      pair = pair_rows;
+    } else {
+      int prev = t > first ? ids[t - 1] : last_id[entry_slot[b]];
+      if (prev < 0 || prev >= V) prev = 0;
+      pair = ((long long)prev * mul_prev + (long long)id * mul_cur) % pair_rows;
+      if (pair < 0) pair += pair_rows;
+    }
+    if (t == first) {
+      __syncthreads();          // every thread of this block has read the old id
+      if (threadIdx.x == 0) last_id[entry_slot[b]] = ids[q_start[b + 1] - 1];
+    }
+  }
+  const T* tok = token_table + (size_t)id * H;
+  const T* pr = pair >= 0 ? pair_table + (size_t)pair * H : nullptr;
+  const float* ps = position_table ? position_table + (size_t)(pos < position_rows ? pos : position_rows - 1) * H : nullptr;
+  float* out = stream + (size_t)t * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    float v = known ? ld_f32(tok + i) * scale : 0.f;
+    if (pr) v += ld_f32(pr + i);
+    if (ps) v += ps[i];
+    out[i] = v;
+  }
+}
+
+extern "C" int ullm_embedding_sum(const int* ids, const void* token_table, float scale, const void* pair_table,
+                                  long long pair_rows, long long mul_prev, long long mul_cur,
+                                  const float* position_table, int position_rows, const int* positions,
+                                  const int* token_entry, const int* q_start, const int* entry_slot, int* last_id,
+                                  float* stream, int T_, int H, int V, int dtype, hipStream_t stream_) {
+  if (T_ <= 0) return 0;
+  if (H <= 0 || V <= 0 || (pair_table && (pair_rows <= 0 || !last_id)) || (position_table && position_rows <= 0))
+    return ULLM_ERR_SHAPE;
+#define GO(TT) hipLaunchKernelGGL(embedding_sum_kernel<TT>, dim3(T_), dim3(256), 0, stream_, ids, (const TT*)token_table, \
+    scale, (const TT*)pair_table, pair_rows, mul_prev, mul_cur, position_table, position_rows, positions, token_entry, \
+    q_start, entry_slot, last_id, stream, H, V)
+  if (dtype == ULLM_F32) GO(float);
+  else if (dtype == ULLM_BF16) GO(bf16_t);
+  else return ULLM_ERR_DTYPE;
+#undef GO
+  ULLM_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------------------------ add + norm, general form
+// For output row r (input row i = rows ? rows[r] : r), with norm_k(v) = (v - mean_k(v)) / sqrt(mean((v - mean_k(v))^2) + eps)
+// where mean_k is the mean for kind 1 (layer norm, no bias) and 0 for kind 0 (RMS norm):
+//   b = float(branch[i])                                   (branch may be null: nothing is added)
+//   if post_gain: b = norm_post_kind(b) * post_gain        (a norm on the branch before it joins the stream)
+//   s = residual[i] + mult * b;  if write_res: residual[i] = s
+//   if y: y[r] = norm_kind(s) * gain
+// One block per row; the row is held in shared memory (H floats) and every thread keeps to its own
+// columns, so the sums have one fixed order whatever else is in the batch.
+template <typename TB, typename TY>
+__global__ void __launch_bounds__(256)
+add_norm_general_kernel(const TB* __restrict__ branch, float* __restrict__ residual,
+                        const float* __restrict__ post_gain, float post_eps, int post_kind, float mult,
+                        const float* __restrict__ gain, float eps, int kind, TY* __restrict__ y,
+                        const int* __restrict__ rows, int H, int write_res) {
+  extern __shared__ float row[];
+  __shared__ float scratch[16];
+  const int r = blockIdx.x;
+  const int i = rows ? rows[r] : r;
+  float* res = residual + (size_t)i * H;
+  const float inv_h = 1.f / (float)H;
+  if (branch) {
+    const TB* br = branch + (size_t)i * H;
+    float sum = 0.f;
+    for (int c = threadIdx.x; c < H; c += blockDim.x) {
+      const float v = ld_f32(br + c);
+      row[c] = v;
+      sum += v;
+    }
+    if (post_gain) {
+      const float mean = post_kind == 1 ? block_sum(sum, scratch) * inv_h : 0.f;
+      float ss = 0.f;
+      for (int c = threadIdx.x; c < H; c += blockDim.x) {
+        const float d = row[c] - mean;
+        ss += d * d;
+      }
+      const float rs = 1.f / sqrtf(block_sum(ss, scratch) * inv_h + post_eps);
+      for (int c = threadIdx.x; c < H; c += blockDim.x) row[c] = ((row[c] - mean) * rs) * post_gain[c];
+    }
+    for (int c = threadIdx.x; c < H; c += blockDim.x) {
+      const float s = res[c] + mult * row[c];
+      if (write_res) res[c] = s;
+      row[c] = s;
+    }
+  } else {
+    for (int c = threadIdx.x; c < H; c += blockDim.x) row[c] = res[c];
+  }
+  if (!y) return;
+  float sum = 0.f;
+  if (kind == 1)
+    for (int c = threadIdx.x; c < H; c += blockDim.x) sum += row[c];
+  const float mean = kind == 1 ? block_sum(sum, scratch) * inv_h : 0.f;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < H; c += blockDim.x) {
+    const float d = row[c] - mean;
+    ss += d * d;
+  }
+  const float rs = 1.f / sqrtf(block_sum(ss, scratch) * inv_h + eps);
+  TY* out = y + (size_t)r * H;
+  for (int c = threadIdx.x; c < H; c += blockDim.x) st_f32(out + c, ((row[c] - mean) * rs) * gain[c]);
+}
+
+extern "C" int ullm_add_norm_general(const void* branch, float* residual, const float* post_gain, float post_eps,
+                                     int post_kind, float mult, const float* gain, float eps, int kind, void* y,
+                                     const int* rows, int n_rows, int H, int branch_dtype, int y_dtype, int write_res,
+                                     hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (H <= 0 || H > 16384 || (kind != 0 && kind != 1) || (post_kind != 0 && post_kind != 1) || (y && !gain))
+    return ULLM_ERR_SHAPE;
+  const size_t shared = (size_t)H * sizeof(float);
+#define GO(TB, TY) hipLaunchKernelGGL((add_norm_general_kernel<TB, TY>), dim3(n_rows), dim3(256), shared, stream, \
+    (const TB*)branch, residual, post_gain, post_eps, post_kind, mult, gain, eps, kind, (TY*)y, rows, H, write_res)
+  if (branch_dtype == ULLM_F32 && y_dtype == ULLM_F32) GO(float, float);
+  else if (branch_dtype == ULLM_BF16 && y_dtype == ULLM_BF16) GO(bf16_t, bf16_t);
+  else if (branch_dtype == ULLM_F32 && y_dtype == ULLM_BF16) GO(float, bf16_t);
+  else if (branch_dtype == ULLM_BF16 && y_dtype == ULLM_F32) GO(bf16_t, float);
+  else return ULLM_ERR_DTYPE;
+#undef GO
+  ULLM_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------------------------ q/k norm over the whole projection + cache write
+// proj[t] holds q at column q_off (nq * hd values), and with has_kv k at k_off and v at v_off (nkv * hd each).
+// q (and k) are divided by the root mean square taken over ALL their values of the token at once
+// (sum of squares / q_count resp. k_count: the counts are given, so that columns a caller padded with
+// zeros do not enter the mean), times a gain per value.  q goes to q_out [T, nq*hd]; k and v go to the
+// paged pools (keys [page, kv_head, row, hd], values [page, kv_head, hd, row]); tokens without a page
+// are not written.  One block per token.
+template <typename T>
+__global__ void __launch_bounds__(256)
+qk_whole_norm_write_kernel(const T* __restrict__ proj, int proj_stride, int q_off, int k_off, int v_off,
+                           T* __restrict__ q_out, int q_out_stride, const float* __restrict__ q_gain,
+                           const float* __restrict__ k_gain, float eps, float q_count, float k_count,
+                           const int* __restrict__ positions, const int* __restrict__ token_entry,
+                           const int* __restrict__ block_table, int bt_stride, T* __restrict__ k_pool,
+                           T* __restrict__ v_pool, int page_size, int nq, int nkv, int hd, int has_kv) {
+  __shared__ float scratch[16];
+  const int t = blockIdx.x;
+  const T* src = proj + (size_t)t * proj_stride;
+  const int nqv = nq * hd;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < nqv; c += blockDim.x) {
+    const float x = ld_f32(src + q_off + c);
+    ss += x * x;
+  }
+  float rs = 1.f;
+  if (q_gain) rs = 1.f / sqrtf(block_sum(ss, scratch) / q_count + eps);
+  T* qo = q_out + (size_t)t * q_out_stride;
+  for (int c = threadIdx.x; c < nqv; c += blockDim.x) {
+    const float x = ld_f32(src + q_off + c);
+    st_f32(qo + c, q_gain ? (x * rs) * q_gain[c] : x);
+  }
+  if (!has_kv) return;
+  const int pos = positions[t];
+  const int page = block_table[(size_t)token_entry[t] * bt_stride + pos / page_size];
+  if (page < 0) return;
+  const int nkvv = nkv * hd;
+  ss = 0.f;
+  for (int c = threadIdx.x; c < nkvv; c += blockDim.x) {
+    const float x = ld_f32(src + k_off + c);
+    ss += x * x;
+  }
+  rs = 1.f;
+  if (k_gain) rs = 1.f / sqrtf(block_sum(ss, scratch) / k_count + eps);
+  const int slot = pos % page_size;
+  for (int c = threadIdx.x; c < nkvv; c += blockDim.x) {
+    const int kvh = c / hd, i = c % hd;
+    const float x = ld_f32(src + k_off + c);
+    st_f32(k_pool + (((size_t)page * nkv + kvh) * page_size + slot) * hd + i, k_gain ? (x * rs) * k_gain[c] : x);
+    v_pool[(((size_t)page * nkv + kvh) * hd + i) * page_size + slot] = src[v_off + c];
+  }
+}
+
+extern "C" int ullm_qk_whole_norm_write(const void* proj, int proj_stride, int q_off, int k_off, int v_off, void* q_out,
+                                        int q_out_stride, const float* q_gain, const float* k_gain, float eps,
+                                        float q_count, float k_count, const int* positions, const int* token_entry,
+                                        const int* block_table, int bt_stride, void* k_pool, void* v_pool,
+                                        int page_size, int T_, int nq, int nkv, int hd, int has_kv, int dtype,
+                                        hipStream_t stream) {
+  if (T_ <= 0) return 0;
+  if (hd <= 0 || nq <= 0 || nkv <= 0 || page_size <= 0 || q_count <= 0.f || k_count <= 0.f) return ULLM_ERR_SHAPE;
+  if (has_kv && (!k_pool || !v_pool)) return ULLM_ERR_SHAPE;
+#define GO(TT) hipLaunchKernelGGL(qk_whole_norm_write_kernel<TT>, dim3(T_), dim3(256), 0, stream, (const TT*)proj, \
+    proj_stride, q_off, k_off, v_off, (TT*)q_out, q_out_stride, q_gain, k_gain, eps, q_count, k_count, positions, \
+    token_entry, block_table, bt_stride, (TT*)k_pool, (TT*)v_pool, page_size, nq, nkv, hd, has_kv)
+  if (dtype == ULLM_F32) GO(float);
+  else if (dtype == ULLM_BF16) GO(bf16_t);
+  else return ULLM_ERR_DTYPE;
+#undef GO
+  ULLM_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------------------------ a gate per head
+// x[t, h*hd + i] *= sigmoid(gate[t*gate_stride + h]) for x [T, nq*hd]; the gate's logistic in 32-bit.
+template <typename T>
+__global__ void head_gate_kernel(T* __restrict__ x, const T* __restrict__ gate, int gate_stride, int nq, int hd, size_t total) {
+  const size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= total) return;
+  const size_t t = e / ((size_t)nq * hd);
+  const int h = (int)((e / hd) % nq);
+  const float g = ld_f32(gate + t * gate_stride + h);
+  st_f32(x + e, ld_f32(x + e) * (1.f / (1.f + expf(-g))));
+}
+
+extern "C" int ullm_head_gate(void* x, const void* gate, int gate_stride, int T_, int nq, int hd, int dtype,
+                              hipStream_t stream) {
+  if (T_ <= 0) return 0;
+  if (nq <= 0 || hd <= 0 || gate_stride < nq) return ULLM_ERR_SHAPE;
+  const size_t total = (size_t)T_ * nq * hd;
+  const unsigned blocks = (unsigned)((total + 255) / 256);
+#define GO(TT) hipLaunchKernelGGL(head_gate_kernel<TT>, dim3(blocks), dim3(256), 0, stream, (TT*)x, (const TT*)gate, \
+    gate_stride, nq, hd, total)
+  if (dtype == ULLM_F32) GO(float);
+  else if (dtype == ULLM_BF16) GO(bf16_t);
+  else return ULLM_ERR_DTYPE;
+#undef GO
+  ULLM_LAUNCH_CHECK();
+}

@@ -262,12 +262,225 @@ def qk_norm_rope_write(qkv: torch.Tensor, q_out: torch.Tensor, q_gain: Optional[
         _c_int(_dt(qkv)), _stream()), "qk_norm_rope_write")
 
 
+
+def scale_(x: torch.Tensor, s: float) -> torch.Tensor:
+    """x *= s in place, float32 [rows, cols]."""
+    _need(x.dtype == torch.float32 and x.dim() == 2 and x.stride(1) == 1, "scale_ takes float32 [rows, cols]")
+    _check(build.load("elementwise").ullm_scale(_p(x), _c_int(x.shape[0]), _c_int(x.shape[1]), _c_int(x.stride(0)),
+                                                _c_float(s), _stream()), "scale")
+    return x
+
+
+def embedding_sum(ids: torch.Tensor, table: torch.Tensor, scale: float, pair_table: Optional[torch.Tensor],
+                  mul_prev: int, mul_cur: int, position_table: Optional[torch.Tensor], positions: torch.Tensor,
+                  token_entry: torch.Tensor, q_start: torch.Tensor, entry_slot: torch.Tensor,
+                  last_id: Optional[torch.Tensor]) -> torch.Tensor:
+    """float32 [T, H]: ``scale`` * table[ids] + pair_table[row] + position_table[positions].  ``pair_table``
+    [buckets + 1, H] is read at (previous id * mul_prev + id * mul_cur) mod buckets, at row ``buckets`` for a
+    request's first token; the id before an entry's first token comes from ``last_id`` (int32 [slots, 1], row =
+    the entry's slot), where the entry's last id is left afterwards.  Either table may be None."""
+    T = ids.numel()
+    V, H = table.shape
+    _i32(ids, "ids")
+    _i32(positions, "positions", T)
+    _i32(token_entry, "token_entry", T)
+    _i32(q_start, "q_start")
+    _i32(entry_slot, "entry_slot")
+    _need(table.is_contiguous(), "embedding table must be contiguous")
+    pair_rows = 0
+    if pair_table is not None:
+        _need(pair_table.is_contiguous() and pair_table.dim() == 2 and pair_table.shape[1] == H
+              and pair_table.dtype == table.dtype and pair_table.shape[0] >= 2, "pair table must be [buckets + 1, H]")
+        _need(last_id is not None and last_id.dtype == torch.int32 and last_id.is_contiguous()
+              and last_id.numel() == last_id.shape[0], "last_id must be contiguous int32 [slots, 1]")
+        pair_rows = pair_table.shape[0] - 1
+    if position_table is not None:
+        _need(position_table.dtype == torch.float32 and position_table.is_contiguous() and position_table.dim() == 2
+              and position_table.shape[1] == H, "position table must be float32 [positions, H]")
+    out = torch.empty((T, H), dtype=torch.float32, device=table.device)
+    ll = ctypes.c_longlong
+    _check(build.load("elementwise").ullm_embedding_sum(
+        _p(ids), _p(table), _c_float(scale), _p(pair_table), ll(pair_rows), ll(int(mul_prev)), ll(int(mul_cur)),
+        _p(position_table), _c_int(0 if position_table is None else position_table.shape[0]), _p(positions),
+        _p(token_entry), _p(q_start), _p(entry_slot), _p(last_id), _p(out), _c_int(T), _c_int(H), _c_int(V),
+        _c_int(_dt(table)), _stream()), "embedding_sum")
+    return out
+
+
+NORM_RMS, NORM_LAYER = 0, 1       # kinds of norm the general add + norm kernel knows
+
+
+def add_norm_general(branch: Optional[torch.Tensor], residual: torch.Tensor, gain: Optional[torch.Tensor], eps: float,
+                     kind: int, out_dtype: Optional[torch.dtype], rows: Optional[torch.Tensor] = None,
+                     post_gain: Optional[torch.Tensor] = None, post_eps: float = 0.0, post_kind: int = NORM_RMS,
+                     mult: float = 1.0) -> Optional[torch.Tensor]:
+    """residual (float32 [T, H], in place unless ``rows``) += mult * b, where b is ``branch`` [T, H] or, with
+    ``post_gain``, the norm of the branch (``post_kind``, ``post_eps``) times that gain; returns the norm
+    (``kind``: NORM_RMS or NORM_LAYER, the layer norm without a bias) of the sum times ``gain`` in ``out_dtype``,
+    or None with ``gain`` None (then only the stream is updated).  Everything is computed in 32-bit."""
+    T, H = residual.shape
+    _need(residual.dtype == torch.float32 and residual.is_contiguous(), "residual must be contiguous float32")
+    for g, nm in ((gain, "gain"), (post_gain, "post_gain")):
+        if g is not None:
+            _need(g.dtype == torch.float32 and g.numel() == H and g.is_contiguous(), f"{nm} must be float32 [H]")
+    if branch is not None:
+        _need(branch.shape == (T, H) and branch.is_contiguous(), "branch must be contiguous [T, H]")
+    n = T
+    if rows is not None:
+        _i32(rows, "rows")
+        n = rows.numel()
+    out = None
+    if gain is not None:
+        out = torch.empty((n, H), dtype=out_dtype, device=residual.device)
+    bdt = _dt(branch) if branch is not None else F32
+    _check(build.load("elementwise").ullm_add_norm_general(
+        _p(branch), _p(residual), _p(post_gain), _c_float(post_eps), _c_int(post_kind), _c_float(mult), _p(gain),
+        _c_float(eps), _c_int(kind), _p(out), _p(rows), _c_int(n), _c_int(H), _c_int(bdt),
+        _c_int(_dt(out) if out is not None else F32), _c_int(0 if rows is not None else 1), _stream()), "add_norm_general")
+    return out
+
+
+def qk_whole_norm_write(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, q_out: torch.Tensor,
+                        q_gain: Optional[torch.Tensor], k_gain: Optional[torch.Tensor], eps: float, q_count: int,
+                        k_count: int, positions: torch.Tensor, token_entry: torch.Tensor, block_table: torch.Tensor,
+                        k_pool: Optional[torch.Tensor], v_pool: Optional[torch.Tensor], page_size: int, nq: int,
+                        nkv: int, hd: int, has_kv: bool) -> None:
+    """q (columns ``q_off``.. of ``proj``, nq*hd values) and, with ``has_kv``, k (``k_off``.., nkv*hd values) are
+    divided by the root mean square over all their values of a token at once (sum of squares / ``q_count`` resp.
+    ``k_count``, eps inside the root) and multiplied by a gain per value (float32 [nq*hd], [nkv*hd]; None: no norm);
+    q goes to ``q_out`` [T, nq*hd], k and v (``v_off``..) to the paged pools."""
+    T = proj.shape[0]
+    width = proj.shape[1]
+    _need(proj.dim() == 2 and proj.stride(1) == 1, "proj must be [T, columns]")
+    _need(0 <= q_off and q_off + nq * hd <= width, "q columns outside the projection")
+    _need(q_out.shape == (T, nq * hd) and q_out.is_contiguous() and q_out.dtype == proj.dtype, "bad q_out")
+    _i32(positions, "positions", T)
+    _i32(token_entry, "token_entry", T)
+    _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.stride(1) == 1,
+          "block_table must be int32 [B, stride]")
+    for g, nm, n in ((q_gain, "q_gain", nq * hd), (k_gain, "k_gain", nkv * hd)):
+        if g is not None:
+            _need(g.dtype == torch.float32 and g.numel() == n and g.is_contiguous(), f"{nm} must be float32 [{n}]")
+    if has_kv:
+        _need(0 <= k_off and k_off + nkv * hd <= width and 0 <= v_off and v_off + nkv * hd <= width,
+              "k or v columns outside the projection")
+        _check_pools(k_pool, v_pool, nkv, page_size, hd, proj.dtype)
+    _check(build.load("elementwise").ullm_qk_whole_norm_write(
+        _p(proj), _c_int(proj.stride(0)), _c_int(q_off), _c_int(k_off), _c_int(v_off), _p(q_out), _c_int(q_out.stride(0)),
+        _p(q_gain), _p(k_gain), _c_float(eps), _c_float(float(q_count)), _c_float(float(k_count)), _p(positions),
+        _p(token_entry), _p(block_table), _c_int(block_table.stride(0)), _p(k_pool if has_kv else None),
+        _p(v_pool if has_kv else None), _c_int(page_size), _c_int(T), _c_int(nq), _c_int(nkv), _c_int(hd),
+        _c_int(1 if has_kv else 0), _c_int(_dt(proj)), _stream()), "qk_whole_norm_write")
+
+
+def head_gate_(x: torch.Tensor, gate: torch.Tensor, nq: int, hd: int) -> torch.Tensor:
+    """x [T, nq*hd] *= sigmoid(gate [T, >= nq])[:, head] in place (``gate`` may be columns of a wider row)."""
+    T = x.shape[0]
+    _need(x.shape == (T, nq * hd) and x.is_contiguous(), "x must be contiguous [T, nq*hd]")
+    _need(gate.dim() == 2 and gate.shape[0] == T and gate.shape[1] >= nq and gate.stride(1) == 1 and gate.dtype == x.dtype,
+          "gate must be [T, >= nq] of x's dtype")
+    _check(build.load("elementwise").ullm_head_gate(_p(x), _p(gate), _c_int(gate.stride(0)), _c_int(T), _c_int(nq),
+                                                    _c_int(hd), _c_int(_dt(x)), _stream()), "head_gate")
+    return x
+
+
+# ---------------------------------------------------------------------------------- recurrent mixers
+
+CONV_MAX_TAPS = 16
+
+
+def conv_silu(proj: torch.Tensor, in_off: int, channels: int, weight: torch.Tensor, bias: Optional[torch.Tensor],
+              carry: torch.Tensor, token_entry: torch.Tensor, q_start: torch.Tensor, entry_slot: torch.Tensor,
+              n_entries: int, update_carry: bool = True) -> torch.Tensor:
+    """silu of a causal convolution per channel over each entry's tokens: float32 [T, channels] from columns
+    ``in_off``.. of ``proj`` (float32 [T, columns]), ``weight`` float32 [channels, taps] (the last column is the
+    current token's), ``bias`` float32 [channels].  ``carry`` (float32 [slots, >= (taps-1)*channels]; may be a view
+    of wider rows) holds the inputs of the taps-1 tokens before the step in the entry's slot row and takes those
+    of the entry's last tokens afterwards."""
+    T = proj.shape[0]
+    _need(proj.dtype == torch.float32 and proj.dim() == 2 and proj.stride(1) == 1, "proj must be float32 [T, columns]")
+    _need(weight.dtype == torch.float32 and weight.dim() == 2 and weight.shape[0] == channels and weight.is_contiguous(),
+          "conv weight must be contiguous float32 [channels, taps]")
+    taps = weight.shape[1]
+    _need(1 <= taps <= CONV_MAX_TAPS, f"a convolution of {taps} taps: at most {CONV_MAX_TAPS}")
+    _need(in_off >= 0 and in_off + channels <= proj.shape[1], "convolution channels outside the projection")
+    if bias is not None:
+        _need(bias.dtype == torch.float32 and bias.numel() == channels and bias.is_contiguous(), "conv bias must be float32 [channels]")
+    _need(carry.dtype == torch.float32 and carry.dim() == 2 and carry.stride(1) == 1
+          and carry.shape[1] >= (taps - 1) * channels, "carry must be float32 [slots, >= (taps-1)*channels]")
+    _i32(token_entry, "token_entry", T)
+    _i32(q_start, "q_start", n_entries + 1)
+    _i32(entry_slot, "entry_slot", n_entries)
+    out = torch.empty((T, channels), dtype=torch.float32, device=proj.device)
+    _check(build.load("recurrent").ullm_conv_silu(
+        _p(proj), _c_int(proj.stride(0)), _c_int(in_off), _p(weight), _p(bias), _p(carry), ctypes.c_longlong(carry.stride(0)),
+        _p(token_entry), _p(q_start), _p(entry_slot), _p(out), _c_int(T), _c_int(n_entries), _c_int(channels), _c_int(taps),
+        _c_int(1 if update_carry else 0), _stream()), "conv_silu")
+    return out
+
+
+def ssm_scan(xbc: torch.Tensor, proj: torch.Tensor, dt_off: int, dt_bias: torch.Tensor, a_log: torch.Tensor,
+             d_skip: torch.Tensor, state: torch.Tensor, state_off: int, q_start: torch.Tensor, entry_slot: torch.Tensor,
+             n_entries: int, heads: int, groups: int, n_state: int, head_dim: int, write_state: bool = True) -> torch.Tensor:
+    """The selective state-space recurrence over each entry's tokens: per head h with state S [n_state, head_dim]
+    (float32, at ``state[slot, state_off + h * n_state * head_dim ..]``), dt = softplus(proj[t, dt_off + h] + dt_bias[h]),
+    S = exp(-exp(a_log[h]) dt) S + dt B x^T, y = S^T C + d_skip[h] x, with x | B | C the columns of ``xbc``
+    (float32 [T, heads*head_dim + 2*groups*n_state]).  Returns y float32 [T, heads*head_dim]."""
+    T = xbc.shape[0]
+    channels = heads * head_dim + 2 * groups * n_state
+    _need(xbc.dtype == torch.float32 and xbc.shape == (T, channels) and xbc.is_contiguous(), "xbc must be contiguous float32 [T, x|B|C]")
+    _need(proj.dtype == torch.float32 and proj.dim() == 2 and proj.stride(1) == 1 and proj.shape[0] == T
+          and 0 <= dt_off and dt_off + heads <= proj.shape[1], "proj must be float32 [T, columns] with the dt columns inside")
+    for v, nm in ((dt_bias, "dt_bias"), (a_log, "a_log"), (d_skip, "d_skip")):
+        _need(v.dtype == torch.float32 and v.numel() == heads and v.is_contiguous(), f"{nm} must be float32 [heads]")
+    _need(state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1
+          and state_off >= 0 and state_off + heads * n_state * head_dim <= state.shape[1], "state must be float32 [slots, row] holding the heads' states")
+    _need(heads % groups == 0 and head_dim <= 256, "heads must be a multiple of groups and head_dim at most 256")
+    _i32(q_start, "q_start", n_entries + 1)
+    _i32(entry_slot, "entry_slot", n_entries)
+    y = torch.empty((T, heads * head_dim), dtype=torch.float32, device=xbc.device)
+    ll = ctypes.c_longlong
+    _check(build.load("recurrent").ullm_ssm_scan(
+        _p(xbc), _p(proj), _c_int(proj.stride(0)), _c_int(dt_off), _p(dt_bias), _p(a_log), _p(d_skip), _p(state),
+        ll(state.stride(0)), ll(state_off), _p(q_start), _p(entry_slot), _p(y), _c_int(n_entries), _c_int(heads),
+        _c_int(groups), _c_int(n_state), _c_int(head_dim), _c_int(1 if write_state else 0), _stream()), "ssm_scan")
+    return y
+
+
+def gated_group_norm(y: torch.Tensor, proj: torch.Tensor, z_off: int, gain: torch.Tensor, eps: float, parts: int,
+                     out_dtype: torch.dtype) -> torch.Tensor:
+    """(y * silu(z)) cut into ``parts`` equal parts, each divided by its own root mean square (eps inside the root),
+    times ``gain``: y float32 [T, width], z = columns ``z_off``.. of ``proj`` (float32), result in ``out_dtype``."""
+    T, width = y.shape
+    _need(y.dtype == torch.float32 and y.is_contiguous(), "y must be contiguous float32")
+    _need(proj.dtype == torch.float32 and proj.dim() == 2 and proj.stride(1) == 1 and proj.shape[0] == T
+          and 0 <= z_off and z_off + width <= proj.shape[1], "proj must be float32 [T, columns] with the gate columns inside")
+    _need(gain.dtype == torch.float32 and gain.numel() == width and gain.is_contiguous(), "gain must be float32 [width]")
+    _need(parts >= 1 and width % parts == 0, f"{width} values do not cut into {parts} equal parts")
+    out = torch.empty((T, width), dtype=out_dtype, device=y.device)
+    _check(build.load("recurrent").ullm_gated_group_norm(
+        _p(y), _p(proj), _c_int(proj.stride(0)), _c_int(z_off), _p(gain), _c_float(eps), _p(out), _c_int(T), _c_int(width),
+        _c_int(parts), _c_int(_dt(out)), _stream()), "gated_group_norm")
+    return out
+
+
 # ---------------------------------------------------------------------------------- attention
+
+def _check_distance_bias(bias: Optional[torch.Tensor], nq: int) -> int:
+    """Rows of a distance-bias table (0 for none) after checking that it is float32 [nq, rows]."""
+    if bias is None:
+        return 0
+    _need(bias.dtype == torch.float32 and bias.dim() == 2 and bias.shape[0] == nq and bias.shape[1] >= 1
+          and bias.is_contiguous(), f"a distance bias must be contiguous float32 [{nq}, rows]")
+    return bias.shape[1]
+
 
 def paged_attention_generic(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
                             positions: torch.Tensor, token_entry: torch.Tensor, block_table: torch.Tensor,
                             page_size: int, nq: int, nkv: int, hd: int, scale: float, window: int,
-                            out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                            out: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``bias`` (float32 [nq, rows]): bias[h, min(distance, rows - 1)] is added to the scaled score of a key
+    ``distance`` positions behind the query."""
     T = q.shape[0]
     _need(q.shape == (T, nq * hd) and q.stride(1) == 1, "q must be [T, nq*hd]")
     _need(hd <= 512 and nq % nkv == 0, "head_dim > 512 or heads not a multiple of kv heads")
@@ -283,7 +496,8 @@ def paged_attention_generic(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch
     _check(lib.ullm_paged_attention_generic(
         _p(q), _c_int(q.stride(0)), _p(out), _c_int(out.stride(0)), _p(k_pool), _p(v_pool), _p(positions),
         _p(token_entry), _p(block_table), _c_int(block_table.stride(0)), _c_int(page_size), _c_int(T),
-        _c_int(nq), _c_int(nkv), _c_int(hd), _c_float(scale), _c_int(window), _c_int(_dt(q)), _stream()),
+        _c_int(nq), _c_int(nkv), _c_int(hd), _c_float(scale), _c_int(window), _p(bias),
+        _c_int(_check_distance_bias(bias, nq)), _c_int(_dt(q)), _stream()),
         "paged_attention_generic")
     return out
 
@@ -734,18 +948,19 @@ def _warn_general_attention(hd: int, page_size: int) -> None:
 
 
 def paged_attention(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, ctx, group, nq: int,
-                    nkv: int, hd: int, scale: float, window: int, plan=None) -> torch.Tensor:
+                    nkv: int, hd: int, scale: float, window: int, plan=None,
+                    bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention of the batch's queries over their requests' cached keys and values (the new
     tokens' rows included).  bfloat16 shapes the matrix-core kernels take go there (one launch for
     the one-token entries, one for the tiles of longer entries, both listed in ``plan``: arrays
     ``decode_tokens`` and ``tiles``, numbers ``num_decode``, ``max_decode_kv``, ``num_tiles``,
     ``tile_keys_total``, ``tile_keys_max``); everything else, and float32 always, takes the general
     kernel.  Every choice computes the same function."""
-    if not attention_mfma_supports(q.dtype, hd, group.page_size, nq, nkv):
-        if q.dtype == torch.bfloat16:
+    if bias is not None or not attention_mfma_supports(q.dtype, hd, group.page_size, nq, nkv):
+        if q.dtype == torch.bfloat16 and bias is None:
             _warn_general_attention(hd, group.page_size)
         return paged_attention_generic(q, k_pool, v_pool, ctx.positions, ctx.token_entry, group.block_table,
-                                       group.page_size, nq, nkv, hd, scale, window)
+                                       group.page_size, nq, nkv, hd, scale, window, bias=bias)
     _need(plan is not None, "the matrix-core attention kernels need the step's work lists (a step plan)")
     out = torch.empty((q.shape[0], nq * hd), dtype=q.dtype, device=q.device)
     n = plan.facts

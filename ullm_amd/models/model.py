@@ -19,6 +19,9 @@ from ..parts import (Block, KVNeed, LayerCache, Norm, Part, PartEnv, StateNeed, 
 from ..parts.linear import linear
 
 
+EMBEDDER_CACHE = -1       # the cache id under which an embedder's per-request state is kept
+
+
 @dataclass(frozen=True)
 class Choice:
     """A part chosen by name with its parameters; parameters may themselves be choices."""
@@ -43,6 +46,10 @@ class ModelPlan:
     embedding_scale: float = 1.0             # the token rows are multiplied by this on their way into the stream
     head_bias: Optional[str] = None          # tensor name of a bias [vocab] on the logits, float32
     logit_softcap: float = 0.0               # > 0: logits = cap * tanh(logits / cap)
+    logit_scale: float = 1.0                 # the logits are multiplied by this
+    # An "embedding" part that makes the stream's first rows (several tables, state of its own); it then owns the
+    # token table and ``embedding_weight`` only names it (for a tied head).  None: the plain scaled row gather.
+    embedder: Optional[Choice] = None
     # The order layers run in: (layer, cache id).  A layer may appear more than once (with a cache id
     # of its own each time, or the same one).  The first entry that names a cache id owns that cache
     # and writes it; later entries with the same id only read it, so a layer can read the cache
@@ -59,6 +66,7 @@ class Model:
         self.plan = plan
         self.blocks: List[Block] = [c.build() for c in plan.layers]
         self.final_norm: Norm = plan.final_norm.build()
+        self.embedder = plan.embedder.build() if plan.embedder is not None else None
         self.run_order = plan.order()
         self.cache_owner: Dict[int, int] = {}      # cache id -> index into run_order of its owner
         for idx, (layer, cache_id) in enumerate(self.run_order):
@@ -72,13 +80,15 @@ class Model:
 
     # ------------------------------------------------------------------ weights
     def parts(self):
+        if self.embedder is not None:
+            yield from walk(self.embedder)
         for b in self.blocks:
             yield from walk(b)
         yield from walk(self.final_norm)
 
     def weight_decls(self) -> List[WeightDecl]:
         p = self.plan
-        decls = [WeightDecl(p.embedding_weight, (p.vocab_size, p.hidden_size))]
+        decls = [] if self.embedder is not None else [WeightDecl(p.embedding_weight, (p.vocab_size, p.hidden_size))]
         for part in self.parts():
             decls.extend(part.weights())
         decls.append(WeightDecl(p.head_weight, (p.vocab_size, p.hidden_size),
@@ -102,6 +112,11 @@ class Model:
         Returns (groups, {(cache id, need index): group index}, {(cache id, need index): StateNeed})."""
         keyed: Dict[KVNeed, List[Tuple[int, int]]] = {}
         states: Dict[Tuple[int, int], StateNeed] = {}
+        if self.embedder is not None and self.embedder.cache_need() is not None:
+            need = self.embedder.cache_need()
+            if not isinstance(need, StateNeed):
+                raise TypeError("an embedder keeps fixed-size state per request or nothing")
+            states[(EMBEDDER_CACHE, 0)] = need
         for cache_id, idx in self.cache_owner.items():
             for i, need in enumerate(cache_needs_of(self.blocks[self.run_order[idx][0]])):
                 if isinstance(need, KVNeed):
@@ -131,13 +146,18 @@ class Model:
 
     def num_needs(self, cache_id: int) -> int:
         """How many needs the block that owns this cache declares."""
+        if cache_id == EMBEDDER_CACHE:
+            return 1
         return len(cache_needs_of(self.blocks[self.run_order[self.cache_owner[cache_id]][0]]))
 
     # ------------------------------------------------------------------ forward
     def forward(self, ctx: StepContext, caches: Dict[int, LayerCache], logit_rows: Optional[torch.Tensor]):
         """Runs the batch through every layer of the run order and returns float32 logits
         [len(logit_rows), vocab] (None if no row is wanted)."""
-        residual = ops.embedding(ctx.token_ids, self.embedding, scale=self.plan.embedding_scale)
+        if self.embedder is not None:
+            residual = self.embedder.forward(ctx, caches.get(EMBEDDER_CACHE) or LayerCache())
+        else:
+            residual = ops.embedding(ctx.token_ids, self.embedding, scale=self.plan.embedding_scale)
         pending = None
         for idx, (layer, cache_id) in enumerate(self.run_order):
             cache = caches.get(cache_id)
@@ -156,6 +176,8 @@ class Model:
             return None
         x = self.final_norm.add_norm(pending, residual, rows=logit_rows, out_dtype=ctx.dtype)
         logits = linear(x, self.head, self.head_bias, out_dtype=torch.float32)
+        if self.plan.logit_scale != 1.0:
+            ops.scale_(logits, self.plan.logit_scale)
         if self.plan.logit_softcap > 0:
             ops.softcap_(logits, self.plan.logit_softcap)
         return logits

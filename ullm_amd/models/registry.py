@@ -27,6 +27,10 @@ def register_architecture(name: str, config_from_dict, plan) -> None:
 
 def resolve_architecture(config_dict: Mapping) -> Architecture:
     archs = config_dict.get("architectures") or []
+    if isinstance(archs, str):
+        archs = [archs]
+    if isinstance(config_dict.get("architecture"), str):      # some configurations name one architecture, in the singular
+        archs = list(archs) + [config_dict["architecture"]]
     for a in archs:
         if a in MODEL_REGISTRY:
             return MODEL_REGISTRY[a]

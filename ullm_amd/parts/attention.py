@@ -5,6 +5,15 @@ projection) and ullm/layers/attention.py:279-313 (write k, v to the cache, then 
 Head size is a parameter of its own (qwen3.py:78: not hidden/heads), the q/k norms and the position
 encoding are optional parts, and a window bounds how far back a query looks (0 = everything; the
 reference never windows).
+
+Beyond that form the same mixer takes, each as a parameter of its own: a value size that differs from the
+query/key size (``value_dim``), the q/k norm taken over the whole projection instead of per head
+(``qk_norm="whole"``, gains of the projections' full sizes), a bias on the scores by distance (a position part
+with ``score_bias()``), a gate per head on the heads' outputs (``head_gate``: sigmoid of one more projection of
+the mixer's input), no key/value projections of its own (``own_kv=False``: the layer reads the cache another
+layer writes), and other tensor names (``names``).  Any of these takes the general path below: one projection
+q | k | v | gate, heads padded with zeros to a size the attention kernels take (zero key dims add nothing to a
+score, zero value dims give zero outputs that meet zero columns of the output projection).
 """
 from __future__ import annotations
 
@@ -23,6 +32,20 @@ from .linear import add_into_stream, can_fuse, linear, linear_into_stream, linea
 # With more, its waves fill the chip and the extra work at each wave's start is no longer hidden behind the
 # others' loads: the kernel of its own, which does it for all tokens at once, is then the faster way.
 FUSED_DECODE_MAX_TOKENS = 64
+
+DEFAULT_NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
+                 "q_norm": "q_norm.weight", "k_norm": "k_norm.weight", "gate": "gate_proj.weight"}
+KERNEL_HEAD_SIZES = (32, 64, 96, 128, 256)      # what the matrix-core attention kernels take
+
+
+def padded_head_size(*sizes: int) -> int:
+    """The size heads are stored with in the cache: the smallest the matrix-core kernels take that holds
+    every given size, or the largest given size (made even) where none does."""
+    need = max(sizes)
+    for size in KERNEL_HEAD_SIZES:
+        if size >= need:
+            return size
+    return need + need % 2
 
 
 def plan_attention_step(shape: StepShape) -> StepPlan:
@@ -60,7 +83,24 @@ class GQAttention(Mixer):
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, prefix: str,
                  position: Optional[PositionEncoding] = None, qk_norm_eps: Optional[float] = None,
-                 bias: bool = False, window: int = 0, scale: Optional[float] = None):
+                 bias: bool = False, window: int = 0, scale: Optional[float] = None,
+                 value_dim: Optional[int] = None, qk_norm: str = "head", head_gate: bool = False,
+                 own_kv: bool = True, names: Optional[Dict[str, str]] = None):
+        if qk_norm not in ("head", "whole"):
+            raise ValueError(f"qk_norm={qk_norm!r}: 'head' (per head) or 'whole' (over the whole projection)")
+        self.dim, self.vdim = head_dim, head_dim if value_dim is None else int(value_dim)
+        self.qk_norm, self.head_gate, self.own_kv = qk_norm, bool(head_gate), bool(own_kv)
+        self.names = {**DEFAULT_NAMES, **(names or {})}
+        self.general = (self.vdim != head_dim or qk_norm == "whole" or self.head_gate or not self.own_kv
+                        or names is not None or (position is not None and type(position).score_bias
+                                                 is not PositionEncoding.score_bias))
+        if self.general:
+            if bias:
+                raise ValueError("projection biases are not built for the general attention path")
+            padded = padded_head_size(head_dim, self.vdim)
+            if qk_norm == "head" and qk_norm_eps is not None and padded != head_dim:
+                raise ValueError(f"a per-head norm over heads of {head_dim} stored as {padded}: not built")
+            head_dim = padded
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads are not a multiple of {num_kv_heads} kv heads")
         if head_dim % 2 or head_dim > 512:
@@ -71,7 +111,7 @@ class GQAttention(Mixer):
         self.qk_norm_eps = qk_norm_eps          # None: no per-head norm
         self.bias = bias
         self.window = int(window)
-        self.scale = float(scale) if scale is not None else head_dim ** -0.5   # qwen3.py:81
+        self.scale = float(scale) if scale is not None else self.dim ** -0.5   # qwen3.py:81
         self.w_qkv = self.b_qkv = self.w_o = self.q_gain = self.k_gain = None
 
     def children(self):
@@ -81,6 +121,8 @@ class GQAttention(Mixer):
         return KVNeed(self.nkv, self.hd, self.window)
 
     def weights(self) -> List[WeightDecl]:
+        if self.general:
+            return self._general_weights()
         p, H, hd = self.prefix, self.hidden_size, self.hd
         # q, k and v are used as one matrix with rows q | k | v, as the reference merges them
         # (ullm/layers/linear.py:381-389); the loader puts the three tensors into its rows
@@ -97,6 +139,8 @@ class GQAttention(Mixer):
         return out
 
     def bind(self, tensors: Dict[str, torch.Tensor], env: PartEnv) -> None:
+        if self.general:
+            return self._general_bind(tensors, env)
         p = self.prefix
         self.w_qkv = tensors[f"{p}.qkv_proj.weight"].contiguous()
         self.w_o = tensors[f"{p}.o_proj.weight"].contiguous()
@@ -107,9 +151,13 @@ class GQAttention(Mixer):
             self.k_gain = tensors[f"{p}.k_norm.weight"].contiguous()
 
     def forward(self, x: torch.Tensor, ctx: StepContext, cache: LayerCache) -> torch.Tensor:
+        if self.general:
+            return self._general_forward(x, ctx, cache)
         return linear_into_stream(self._attend(linear(x, self.w_qkv, self.b_qkv), ctx, cache), self.w_o, ctx)
 
     def fusable(self, residual, ctx: StepContext) -> bool:
+        if self.general:
+            return False
         return can_fuse(residual, ctx.dtype, self.w_qkv, self.w_o)
 
     def forward_fused(self, x, residual, ctx: StepContext, cache: LayerCache, then=None):
@@ -144,3 +192,85 @@ class GQAttention(Mixer):
             cache.k_pool, cache.v_pool, group.page_size, self.nq, self.nkv, self.hd, write_kv=cache.owner)
         return ops.paged_attention(q, cache.k_pool, cache.v_pool, ctx, group, self.nq, self.nkv, self.hd,
                                    self.scale, self.window, plan)
+
+    # ------------------------------------------------------------------ the general path
+    def _name(self, role: str) -> str:
+        return f"{self.prefix}.{self.names[role]}"
+
+    def _general_weights(self) -> List[WeightDecl]:
+        H, nq, nkv, d, dv = self.hidden_size, self.nq, self.nkv, self.dim, self.vdim
+        out = [WeightDecl(self._name("q"), (nq * d, H)), WeightDecl(self._name("o"), (H, nq * dv))]
+        if self.own_kv:
+            out += [WeightDecl(self._name("k"), (nkv * d, H)), WeightDecl(self._name("v"), (nkv * dv, H))]
+        if self.qk_norm_eps is not None:
+            per = d if self.qk_norm == "head" else None
+            out.append(WeightDecl(self._name("q_norm"), (per or nq * d,), init="gain", keep_fp32=True))
+            if self.own_kv:
+                out.append(WeightDecl(self._name("k_norm"), (per or nkv * d,), init="gain", keep_fp32=True))
+        if self.head_gate:
+            out.append(WeightDecl(self._name("gate"), (nq, H)))
+        return out
+
+    def _general_bind(self, tensors: Dict[str, torch.Tensor], env: PartEnv) -> None:
+        """One input matrix with rows q | k | v | gate (a reader of another layer's cache: q | gate), every head
+        padded with zero rows to the stored head size, the gate's rows to a multiple of eight; the output
+        matrix with zero columns where the values are padded; gains padded alike."""
+        H, nq, nkv, d, dv, hd = self.hidden_size, self.nq, self.nkv, self.dim, self.vdim, self.hd
+
+        def heads_padded(t: torch.Tensor, heads: int, size: int) -> torch.Tensor:      # [heads*size, ...] -> [heads*hd, ...]
+            if size == hd:
+                return t
+            out = torch.zeros((heads, hd) + tuple(t.shape[1:]), dtype=t.dtype, device=t.device)
+            out[:, :size] = t.view((heads, size) + tuple(t.shape[1:]))
+            return out.view((heads * hd,) + tuple(t.shape[1:]))
+
+        pieces = [heads_padded(tensors[self._name("q")], nq, d)]
+        self.q_off, self.k_off, self.v_off = 0, nq * hd, (nq + nkv) * hd
+        if self.own_kv:
+            pieces += [heads_padded(tensors[self._name("k")], nkv, d), heads_padded(tensors[self._name("v")], nkv, dv)]
+        self.gate_off = sum(p.shape[0] for p in pieces)
+        if self.head_gate:
+            gate = tensors[self._name("gate")]
+            pieces.append(torch.cat((gate, gate.new_zeros((-nq % 8, H))), dim=0))
+        self.w_qkv = torch.cat(pieces, dim=0).contiguous()
+        w_o = tensors[self._name("o")]
+        if dv != hd:
+            wide = w_o.new_zeros((H, nq, hd))
+            wide[:, :, :dv] = w_o.view(H, nq, dv)
+            w_o = wide.view(H, nq * hd)
+        self.w_o = w_o.contiguous()
+        if self.qk_norm_eps is not None:
+            if self.qk_norm == "head":
+                self.q_gain = tensors[self._name("q_norm")].contiguous()
+                self.k_gain = tensors[self._name("k_norm")].contiguous() if self.own_kv else None
+            else:
+                self.q_gain = heads_padded(tensors[self._name("q_norm")], nq, d).contiguous()
+                self.k_gain = heads_padded(tensors[self._name("k_norm")], nkv, d).contiguous() if self.own_kv else None
+
+    def _general_forward(self, x: torch.Tensor, ctx: StepContext, cache: LayerCache) -> torch.Tensor:
+        if cache.owner != self.own_kv:
+            raise RuntimeError(f"{self.prefix}: a layer " + ("with keys and values of its own must write its cache"
+                               if self.own_kv else "without keys and values of its own cannot own a cache"))
+        nq, nkv, hd = self.nq, self.nkv, self.hd
+        T = x.shape[0]
+        group = ctx.groups[cache.group]
+        proj = linear(x, self.w_qkv)
+        q = torch.empty((T, nq * hd), dtype=proj.dtype, device=proj.device)
+        table, rot, style = self.position.kernel_args() if self.position is not None else (None, 0, 0)
+        if self.qk_norm == "head" and self.own_kv:
+            ops.qk_norm_rope_write(proj[:, :(nq + 2 * nkv) * hd], q, self.q_gain, self.k_gain, self.qk_norm_eps or 0.0,
+                                   table, rot, style, ctx.positions, ctx.token_entry, group.block_table, cache.k_pool,
+                                   cache.v_pool, group.page_size, nq, nkv, hd, write_kv=True)
+        else:
+            if style != 0 and rot > 0 or (self.qk_norm == "head" and self.qk_norm_eps is not None):
+                raise NotImplementedError("rotation or a per-head norm without keys of the layer's own: not built")
+            ops.qk_whole_norm_write(proj, self.q_off, self.k_off, self.v_off, q, self.q_gain, self.k_gain,
+                                    self.qk_norm_eps or 0.0, nq * self.dim, nkv * self.dim, ctx.positions,
+                                    ctx.token_entry, group.block_table, cache.k_pool, cache.v_pool, group.page_size,
+                                    nq, nkv, hd, has_kv=self.own_kv)
+        out = ops.paged_attention(q, cache.k_pool, cache.v_pool, ctx, group, nq, nkv, hd, self.scale, self.window,
+                                  ctx.plans["attention"],
+                                  bias=self.position.score_bias() if self.position is not None else None)
+        if self.head_gate:
+            ops.head_gate_(out, proj[:, self.gate_off:], nq, hd)
+        return linear_into_stream(out, self.w_o, ctx)

@@ -3,8 +3,8 @@ and a registry from (kind, name) to the class, so that a model is put together f
 plan that names its parts layer by layer.
 
 Kinds: "mixer" (attention or anything else that mixes tokens), "ffn" (feed-forward),
-"norm", "position" (position encoding) and "block" (how norm, mixer and feed-forward are
-arranged around the residual stream).  No part knows which model it is in: sizes and
+"norm", "position" (position encoding), "block" (how norm, mixer and feed-forward are
+arranged around the residual stream) and "embedding" (how token ids become the stream's first rows).  No part knows which model it is in: sizes and
 constants arrive as constructor parameters, tensor names as a prefix.
 """
 from __future__ import annotations
@@ -31,6 +31,15 @@ class WeightDecl:
     # that already holds the whole matrix under that name is taken as it is.
     merged_into: Optional[str] = None
     row_offset: int = 0
+    # Dimensions whose size the checkpoint decides (a table with as many rows as it was trained with): the
+    # loader accepts any size there and the part reads it off the tensor; ``shape`` holds the size that random
+    # weights are drawn with.
+    free_dims: Tuple[int, ...] = ()
+
+    def fits(self, shape) -> bool:
+        shape = tuple(shape)
+        return len(shape) == len(self.shape) and all(a == b or i in self.free_dims
+                                                     for i, (a, b) in enumerate(zip(shape, self.shape)))
 
 
 # --------------------------------------------------------------------------- cache needs
@@ -298,6 +307,17 @@ class PendingNorm:
         return self.norm.add_norm(None, self.stream, out_dtype=self.out_dtype)
 
 
+@dataclass
+class NormedBranch:
+    """A branch output that joins the stream as ``mult * norm(branch) * gain``: the norm behind a mixer or
+    feed-forward of a block that norms on both sides of each.  It is handed on as the pending branch, and the
+    norm that adds it (``Norm.add_norm``) applies ``post`` (a :class:`Norm` with ``kernel_form()``), the
+    multiplier, the add and its own norm in one pass over the row."""
+    branch: torch.Tensor          # [T, hidden] in the compute dtype
+    post: "Norm"
+    mult: float = 1.0
+
+
 class Norm(Part):
     """``add_norm(branch, residual, rows) -> normed``: adds the branch output (if any) into
     the 32-bit residual stream, then normalises the sum; ``rows`` selects output rows.
@@ -309,6 +329,12 @@ class Norm(Part):
     the stream by, or None if this norm is not a gain times rsqrt(mean of squares + eps)."""
     kind = "norm"
     adds_stacks = False
+
+    def kernel_form(self):
+        """(gain float32 [hidden], eps, kind) with kind one of ``ops.NORM_RMS`` / ``ops.NORM_LAYER`` for a norm that
+        is a gain times the row over its root mean square (after taking the mean off, for a layer norm), or None.
+        A norm with such a form can stand behind a branch (:class:`NormedBranch`)."""
+        return None
 
     def pending(self, residual: torch.Tensor, out_dtype: torch.dtype, scaled: Optional[torch.Tensor] = None,
                 squares: Optional[torch.Tensor] = None) -> Optional["PendingNorm"]:
@@ -330,6 +356,11 @@ class PositionEncoding(Part):
 
     def kernel_args(self):
         return None, 0, 0
+
+    def score_bias(self) -> Optional[torch.Tensor]:
+        """float32 [heads, rows] or None: entry [h, min(distance, rows - 1)] is added to the scaled score of a key
+        ``distance`` positions behind the query (positions that enter the scores rather than the vectors)."""
+        return None
 
 
 class Block(Part):
@@ -357,9 +388,22 @@ class Block(Part):
         raise NotImplementedError
 
 
+class Embedder(Part):
+    """How a step's token ids become the first rows of the residual stream: ``forward(ctx, cache) -> float32
+    [T, hidden]``.  An embedder that needs something of the tokens before the step (the id before an entry's
+    first token) declares a ``StateNeed`` and finds its rows as ``cache.state`` through ``ctx.entry_slot``."""
+    kind = "embedding"
+
+    def cache_need(self) -> CacheNeed:
+        return None
+
+    def forward(self, ctx: StepContext, cache: LayerCache) -> torch.Tensor:
+        raise NotImplementedError
+
+
 # --------------------------------------------------------------------------- registry
 
-_PARTS: Dict[str, Dict[str, Callable]] = {k: {} for k in ("mixer", "ffn", "norm", "position", "block")}
+_PARTS: Dict[str, Dict[str, Callable]] = {k: {} for k in ("mixer", "ffn", "norm", "position", "block", "embedding")}
 
 
 def register_part(kind: str, name: str):

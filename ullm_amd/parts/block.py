@@ -9,7 +9,7 @@ from __future__ import annotations
 
 from typing import Optional
 
-from .base import Block, FeedForward, LayerCache, Mixer, Norm, PendingNorm, StepContext, register_part
+from .base import Block, FeedForward, LayerCache, Mixer, Norm, NormedBranch, PendingNorm, StepContext, register_part
 
 
 @register_part("block", "prenorm")
@@ -65,3 +65,45 @@ class PreNormBlock(Block):
             if record is not None:
                 return record
         return norm.add_norm(pending, residual, out_dtype=ctx.dtype)
+
+
+@register_part("block", "sandwich")
+class SandwichBlock(Block):
+    """Norms on both sides of each sublayer and a multiplier on what joins the stream:
+    h += mult * mixer_post(mixer(mixer_norm(h))); h += mult * ffn_post(ffn(ffn_norm(h))).  A block without a
+    feed-forward (``ffn`` None) has the first sublayer only.  The norm behind a sublayer is not a kernel of
+    its own: the branch is handed on as a :class:`NormedBranch`, and the next norm of the stream applies it,
+    the multiplier, the add and itself in one pass."""
+
+    def __init__(self, mixer_norm: Norm, mixer: Mixer, mixer_post: Norm, mult: float = 1.0,
+                 ffn_norm: Optional[Norm] = None, ffn: Optional[FeedForward] = None, ffn_post: Optional[Norm] = None):
+        if (ffn is None) != (ffn_norm is None) or (ffn is None) != (ffn_post is None):
+            raise ValueError("a feed-forward comes with the norms on both of its sides, or not at all")
+        self.mixer_norm, self.mixer, self.mixer_post = mixer_norm, mixer, mixer_post
+        self.ffn_norm, self.ffn, self.ffn_post = ffn_norm, ffn, ffn_post
+        self.mult = float(mult)
+
+    def children(self):
+        return [p for p in (self.mixer_norm, self.mixer, self.mixer_post, self.ffn_norm, self.ffn, self.ffn_post)
+                if p is not None]
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    def entry_norm(self):
+        return self.mixer_norm
+
+    def forward(self, residual, pending, ctx: StepContext, cache: LayerCache):
+        if isinstance(pending, PendingNorm):
+            pending = None                               # the stream is complete; this block norms it itself
+        x = self.mixer_norm.add_norm(pending, residual, out_dtype=ctx.dtype)
+        pending = NormedBranch(_one_branch(self.mixer.forward(x, ctx, cache)), self.mixer_post, self.mult)
+        if self.ffn is None:
+            return residual, pending
+        x = self.ffn_norm.add_norm(pending, residual, out_dtype=ctx.dtype)
+        return residual, NormedBranch(_one_branch(self.ffn.forward(x, ctx)), self.ffn_post, self.mult)
+
+
+def _one_branch(y):
+    """A stack of partial sums [S, T, hidden] added up: a norm behind the branch needs the whole rows."""
+    return y.sum(0).contiguous() if y.dim() == 3 else y

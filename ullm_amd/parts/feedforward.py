@@ -4,7 +4,7 @@ projection with rows gate | up (qwen3.py:307-308).
 """
 from __future__ import annotations
 
-from typing import Dict, List
+from typing import Dict, List, Optional
 
 import torch
 
@@ -18,21 +18,24 @@ class SwiGLU(FeedForward):
     folds_norm = True
     hands_norm_ahead = True
 
-    def __init__(self, hidden_size: int, intermediate_size: int, prefix: str):
+    def __init__(self, hidden_size: int, intermediate_size: int, prefix: str, names: Optional[Dict[str, str]] = None):
         self.hidden_size, self.intermediate_size, self.prefix = hidden_size, intermediate_size, prefix
+        # tensor names behind the prefix; "gate_up" is the merged matrix's (a checkpoint may hold it whole)
+        self.names = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight",
+                      "gate_up": "gate_up_proj.weight", **(names or {})}
         self.w_gate_up = self.w_down = None
 
     def weights(self) -> List[WeightDecl]:
-        p, H, I = self.prefix, self.hidden_size, self.intermediate_size
-        merged = f"{p}.gate_up_proj.weight"          # rows gate | up, put together by the loader
-        return [WeightDecl(f"{p}.gate_proj.weight", (I, H), merged_into=merged, row_offset=0),
-                WeightDecl(f"{p}.up_proj.weight", (I, H), merged_into=merged, row_offset=I),
-                WeightDecl(f"{p}.down_proj.weight", (H, I))]
+        p, H, I, n = self.prefix, self.hidden_size, self.intermediate_size, self.names
+        merged = f"{p}.{n['gate_up']}"               # rows gate | up, put together by the loader
+        return [WeightDecl(f"{p}.{n['gate']}", (I, H), merged_into=merged, row_offset=0),
+                WeightDecl(f"{p}.{n['up']}", (I, H), merged_into=merged, row_offset=I),
+                WeightDecl(f"{p}.{n['down']}", (H, I))]
 
     def bind(self, tensors: Dict[str, torch.Tensor], env: PartEnv) -> None:
-        p = self.prefix
-        self.w_gate_up = tensors[f"{p}.gate_up_proj.weight"].contiguous()
-        self.w_down = tensors[f"{p}.down_proj.weight"].contiguous()
+        p, n = self.prefix, self.names
+        self.w_gate_up = tensors[f"{p}.{n['gate_up']}"].contiguous()
+        self.w_down = tensors[f"{p}.{n['down']}"].contiguous()
 
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         act = gate_up(x, self.w_gate_up)

@@ -10,11 +10,12 @@ alike that leaves every q.k unchanged, so outputs are kept in place here.
 """
 from __future__ import annotations
 
+import math
 from typing import Dict, Optional
 
 import torch
 
-from .base import PartEnv, PositionEncoding, register_part
+from .base import PartEnv, PositionEncoding, WeightDecl, register_part
 
 
 @register_part("position", "none")
@@ -54,3 +55,55 @@ class Rotary(PositionEncoding):
 
     def kernel_args(self):
         return self.table, self.rotary_dim, self.style
+
+
+def log_distance_bucket(distance: int, rows: int, far: int) -> int:
+    """The table row of a key ``distance`` >= 0 positions behind the query: the distance itself below
+    rows // 2, then rows - rows // 2 further rows spread evenly over the logarithm of the distance up to ``far``,
+    every greater distance in the last row."""
+    half = rows // 2
+    if distance < half:
+        return distance
+    step = math.log(distance / half) / math.log(far / half) * (rows - half)
+    return min(rows - 1, half + int(math.floor(step)))
+
+
+@register_part("position", "log_distance_bias")
+class LogDistanceBias(PositionEncoding):
+    """Positions that enter the scores and not the vectors: a learned table [rows, heads] whose row
+    :func:`log_distance_bucket` of the distance between query and key is added to the scaled score.  For the
+    kernels the table is unrolled by distance once, float32 [heads, distances], up to the first distance
+    that falls into the last row; they clamp greater distances to that entry."""
+
+    DEFAULT_ROWS = 32        # what random weights are drawn with; a checkpoint's table has the rows it has
+
+    def __init__(self, heads: int, far: int, weight_name: str, rows: Optional[int] = None):
+        self.rows = int(rows) if rows is not None else None       # None: read off the bound tensor
+        self.heads, self.far, self.weight_name = int(heads), int(far), weight_name
+        self.by_distance: Optional[torch.Tensor] = None
+
+    def weights(self):
+        if self.rows is None:
+            return [WeightDecl(self.weight_name, (self.DEFAULT_ROWS, self.heads), keep_fp32=True, free_dims=(0,))]
+        return [WeightDecl(self.weight_name, (self.rows, self.heads), keep_fp32=True)]
+
+    def buckets(self) -> list:
+        """Bucket by distance, ending with the first distance in the last row."""
+        out, d = [], 0
+        while True:
+            out.append(log_distance_bucket(d, self.rows, self.far))
+            if out[-1] == self.rows - 1:
+                return out
+            d += 1
+
+    def bind(self, tensors: Dict[str, torch.Tensor], env: PartEnv) -> None:
+        table = tensors[self.weight_name].to(torch.float32)
+        self.rows = table.shape[0]
+        if self.rows < 2 or self.far <= self.rows // 2:
+            raise ValueError(f"{self.weight_name}: a distance table of {self.rows} rows reaching to {self.far}: it needs "
+                             f"two rows and a reach beyond rows // 2")
+        index = torch.tensor(self.buckets(), dtype=torch.long, device=table.device)
+        self.by_distance = table[index].T.contiguous()           # [heads, distances]
+
+    def score_bias(self):
+        return self.by_distance

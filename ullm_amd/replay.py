@@ -28,6 +28,7 @@ def parse_args(argv=None):
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens live requests hold at any time (each rounded up to 64)")
     ap.add_argument("--page-size", type=int, default=16, help="tokens per cache page (divides 64)")
+    ap.add_argument("--max-requests", type=int, default=4, help="request slots: most requests live at any time")
     ap.add_argument("--device", default="cuda:0")
     ap.add_argument("--enforce-eager", action="store_true", help="never replay decode steps from HIP graphs")
     return ap.parse_args(argv)
@@ -90,7 +91,7 @@ def main(argv=None) -> int:
     os.makedirs(args.out, exist_ok=True)
     try:
         rep = Replayer(args.model, args.dtype, args.max_tokens, args.page_size, args.device,
-                       use_graphs=not args.enforce_eager)
+                       max_requests=args.max_requests, use_graphs=not args.enforce_eager)
     except ValueError as e:
         print(f"trace_run: {e}", file=sys.stderr)
         return 2

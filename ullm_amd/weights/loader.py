@@ -98,7 +98,7 @@ def check_against(decls: List[WeightDecl], index) -> None:
     missing, wrong = [], []
     for name, d in declared.items():
         if name in index:
-            if tuple(index[name][1]) != tuple(d.shape):
+            if not d.fits(index[name][1]):
                 wrong.append(f"  {name}  checkpoint has {list(index[name][1])}, model needs {list(d.shape)}")
             continue
         if d.alias_of is not None and d.alias_of in index:
