@@ -103,11 +103,27 @@ __device__ __forceinline__ void load_tile(KVTile<NQK>& t, int key0, const PageWi
 // of from the cache, where the same kernel is only just writing them.
 // INNER: every key of the tile is written data that every column may see (no key before a window's start, none
 // past the newest): no test per score, no zeroing of values, and the token's own key is not in it.
-template <int NQK, int NG, bool OWN, bool INNER>
+// What the variants with EXTRA add to a score and to a head's output: a bias by distance, bias[head][min(query
+// position - key position, last)] in units of log2 (the caller multiplies its table by log2(e) once: the scores
+// are exponents of two), added to the scaled score in 32-bit; and a gate per head, sigmoid(gate[token][head]),
+// that multiplies the head's normalised output on its way out.  Either pointer may be null.
+struct ScoreExtras {
+  const float* bias;          // [nq][bias_rows]
+  int bias_rows;
+  const bf16_t* gate;         // [tokens][gate_stride], one value per head
+  int gate_stride;
+};
+__device__ __forceinline__ float gate_of(const ScoreExtras& x, int token, int head) {
+  if (!x.gate) return 1.f;
+  return 1.f / (1.f + __expf(-bf16_bits_to_f32(x.gate[(size_t)token * x.gate_stride + head])));
+}
+
+template <int NQK, int NG, bool OWN, bool INNER, bool EXTRA = false>
 __device__ __forceinline__ void process_tile(const KVTile<NQK>& cur, int key0, const Pack8 (&qreg)[NG][NQK],
                                              const int (&col_lo)[NG], const int (&col_hi)[NG], int max_hi,
                                              float scale_log2e, f32x4_t (&acc)[NG][2 * NQK], float (&m)[NG],
-                                             float (&l)[NG], const bf16_t* own) {
+                                             float (&l)[NG], const bf16_t* own, const float* bias_col = nullptr,
+                                             int bias_last = 0) {
   // no product fused with a following sum here: the variant with tests keeps the scaled score in a select, the
   // variant without would fuse it into the subtraction of the maximum, and the two would round differently
 #pragma clang fp contract(off)
@@ -172,7 +188,14 @@ __device__ __forceinline__ void process_tile(const KVTile<NQK>& cur, int key0, c
       for (int r = 0; r < 4; ++r) {
         const int kk = key0 + 16 * sb + 4 * g + r;
         const bool ok = INNER || (cur.ok[sb] && kk >= col_lo[q] && kk <= col_hi[q]);
-        const float v = ok ? s[sb][r] * scale_log2e : NEG_BIG;
+        float v = ok ? s[sb][r] * scale_log2e : NEG_BIG;
+        if constexpr (EXTRA) {
+          // the one column of a decode step sits at position max_hi
+          if (bias_col && ok) {
+            const int d = max_hi - kk;
+            v += bias_col[d < bias_last ? (d > 0 ? d : 0) : bias_last];
+          }
+        }
         s[sb][r] = v;
         tile_max = fmaxf(tile_max, v);
       }
@@ -218,12 +241,12 @@ __device__ __forceinline__ void process_tile(const KVTile<NQK>& cur, int key0, c
 // is worked on (two tiles ahead, in three sets of registers, was slower at every batch size and context: the
 // third set costs moves between the two halves of the register file, and a wave's products are the longer
 // part of a tile's time).
-template <int NQK, int NG, bool OWN, class Queries>
+template <int NQK, int NG, bool OWN, class Queries, bool EXTRA = false>
 __device__ __forceinline__ void attend_range(
     Queries& queries, const int (&col_lo)[NG], const int (&col_hi)[NG], int key_begin, int key_end,
     int max_hi, int all_lo, const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
     const int* __restrict__ bt, int page_size, int nkv, int kvh, float scale_log2e, f32x4_t (&acc)[NG][2 * NQK],
-    float (&m)[NG], float (&l)[NG]) {
+    float (&m)[NG], float (&l)[NG], const float* bias_col = nullptr, int bias_last = 0) {
 #pragma unroll
   for (int q = 0; q < NG; ++q) {
 #pragma unroll
@@ -243,9 +266,11 @@ __device__ __forceinline__ void attend_range(
 #define TILE_WORK(T, K0)                                                                                          \
   do {                                                                                                            \
     if ((K0) >= all_lo && (K0) + 31 < max_hi + (OWN ? 0 : 1) && T.ok[0] && T.ok[1])                               \
-      process_tile<NQK, NG, OWN, true>(T, K0, qreg, col_lo, col_hi, max_hi, scale_log2e, acc, m, l, own);         \
+      process_tile<NQK, NG, OWN, true, EXTRA>(T, K0, qreg, col_lo, col_hi, max_hi, scale_log2e, acc, m, l, own,   \
+                                              bias_col, bias_last);                                               \
     else                                                                                                          \
-      process_tile<NQK, NG, OWN, false>(T, K0, qreg, col_lo, col_hi, max_hi, scale_log2e, acc, m, l, own);        \
+      process_tile<NQK, NG, OWN, false, EXTRA>(T, K0, qreg, col_lo, col_hi, max_hi, scale_log2e, acc, m, l, own,  \
+                                               bias_col, bias_last);                                              \
   } while (0)
   KVTile<NQK> t0, t1;                                     // in turns: one is worked on while the other loads
   int base = key_begin, stop = base + 1024 < key_end ? base + 1024 : key_end;
@@ -492,14 +517,14 @@ struct RawQueries {
   }
 };
 
-template <int NQK, int WAVES, bool FUSE>
+template <int NQK, int WAVES, bool FUSE, bool EXTRA = false>
 __global__ void __launch_bounds__(64 * WAVES)
 attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
                         const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
                         const int* __restrict__ token_list, const int* __restrict__ positions,
                         const int* __restrict__ token_entry, const int* __restrict__ block_table,
                         int bt_stride, int page_size, int nq, int nkv, float scale_log2e, int window,
-                        int num_splits, float* __restrict__ part, DecodeFuse fuse) {
+                        int num_splits, float* __restrict__ part, DecodeFuse fuse, ScoreExtras extras) {
   constexpr int HD = 32 * NQK;
   constexpr int ROW = HD + 4;                       // output dims, then maximum and sum (rows stay 16-byte aligned)
   __shared__ float merge[(WAVES > 1 ? WAVES / 2 : 1) * (WAVES > 1 ? (8 * NQK + 2) * 64 : 1)];   // [writer][value][lane]: conflict-free
@@ -552,8 +577,14 @@ attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
         queries.v_dst = fuse.v_pool + ((size_t)page * nkv + kvh) * HD * page_size + off;
       }
     }
-    attend_range<NQK, 1, FUSE>(queries, clo, chi, begin, end, pos, lo, k_pool, v_pool, bt, page_size, nkv, kvh,
-                               scale_log2e, accs, ms, ls);
+    if constexpr (EXTRA) {
+      const float* bias_col = extras.bias ? extras.bias + (size_t)(col_ok ? head : 0) * extras.bias_rows : nullptr;
+      attend_range<NQK, 1, FUSE, Queries, true>(queries, clo, chi, begin, end, pos, lo, k_pool, v_pool, bt, page_size, nkv,
+                                                kvh, scale_log2e, accs, ms, ls, bias_col, extras.bias_rows - 1);
+    } else {
+      attend_range<NQK, 1, FUSE>(queries, clo, chi, begin, end, pos, lo, k_pool, v_pool, bt, page_size, nkv, kvh,
+                                 scale_log2e, accs, ms, ls);
+    }
   }
   merge_waves<NQK, 1, WAVES>(accs, ms, ls, merge);
   f32x4_t (&acc)[2 * NQK] = accs[0];
@@ -564,7 +595,8 @@ attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
   l += __shfl_xor(l, 32, 64);
   if (!col_ok) return;
   if (num_splits == 1) {
-    const float inv = l > 0.f ? 1.f / l : 0.f;
+    float inv = l > 0.f ? 1.f / l : 0.f;
+    if constexpr (EXTRA) inv *= gate_of(extras, t, head);
     bf16_t* op = out + (size_t)t * out_stride + (size_t)head * HD;
 #pragma unroll
     for (int n = 0; n < 2 * NQK; ++n)
@@ -588,7 +620,7 @@ attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
 // its output dims over the splits with the splits' weights passed round by shuffles.
 __global__ void __launch_bounds__(64)
 attention_reduce_kernel(const float* __restrict__ part, bf16_t* __restrict__ out, int out_stride,
-                        const int* __restrict__ token_list, int nq, int hd, int num_splits) {
+                        const int* __restrict__ token_list, int nq, int hd, int num_splits, ScoreExtras extras) {
   const int item = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   const int t = token_list ? token_list[item] : item;
   const int row = hd + 4;
@@ -633,7 +665,7 @@ attention_reduce_kernel(const float* __restrict__ part, bf16_t* __restrict__ out
       }
     }
   }
-  const float inv = L > 0.f ? 1.f / L : 0.f;
+  const float inv = (L > 0.f ? 1.f / L : 0.f) * gate_of(extras, t, head);
   bf16_t* op = out + (size_t)t * out_stride + (size_t)head * hd;
 #pragma unroll
   for (int r = 0; r < 4; ++r)
@@ -800,11 +832,12 @@ __device__ __forceinline__ ScoreScale split_scale(float scale_log2e) {
 // there was none (m == NEG_BIG counts from zero), it becomes the new one, and the exponents and the output so
 // far are brought to it.  Leaves the weights in `p`, rounded to bfloat16 as they multiply the values, and adds
 // those rounded weights to the sums `l`, two per instruction.
-template <int NQK, int NG, bool masked, typename KeyOf>
+template <int NQK, int NG, bool masked, bool EXTRA = false, typename KeyOf>
 __device__ __forceinline__ void prompt_tile_softmax(f32x4_t (&s)[NG][2], int key0, KeyOf key_of,
                                                     const int (&col_lo)[NG], const int (&col_hi)[NG],
                                                     f32x4_t (&acc)[NG][2 * NQK], float (&m)[NG], f32x4_t (&negm)[NG],
-                                                    float (&l)[NG], Pack8 (&p)[NG], const ScoreScale& scale) {
+                                                    float (&l)[NG], Pack8 (&p)[NG], const ScoreScale& scale,
+                                                    const float* bias_row = nullptr, int bias_last = 0) {
   float lane_max[NG], alpha[NG];
   bool exceeds = false;
 #pragma unroll
@@ -816,6 +849,12 @@ __device__ __forceinline__ void prompt_tile_softmax(f32x4_t (&s)[NG][2], int key
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         s[q][sb][r] *= scale.frac;                      // the part of scale * log2(e) that is no power of two, in 32-bit
+        if constexpr (EXTRA) {
+          if (bias_row) {                               // a column's position is the last key it sees
+            const int d = col_hi[q] - (key0 + key_of(sb, r));
+            s[q][sb][r] += bias_row[d < bias_last ? (d > 0 ? d : 0) : bias_last];
+          }
+        }
         if (masked) {
           const int kk = key0 + key_of(sb, r);
           if (!(kk >= col_lo[q] && kk <= col_hi[q])) s[q][sb][r] = NEG_BIG;
@@ -879,12 +918,13 @@ __device__ __forceinline__ void prompt_tile_softmax(f32x4_t (&s)[NG][2], int key
 // starts from minus the column's reference value over the remaining factor (`negm`, the same in all four
 // elements) instead of zero, so the products times that factor are the exponent itself: exp2 of it is the weight.  A column without a reference
 // value yet (m == NEG_BIG) counts from zero, and the first tile that shows it a key gives it one.
-template <int NQK, int NG, bool masked>
+template <int NQK, int NG, bool masked, bool EXTRA = false>
 __device__ __forceinline__ void process_tile_lds(const unsigned char* __restrict__ kl, const unsigned char* __restrict__ vl,
                                                  int key0, const Pack8 (&qreg)[NG][NQK],
                                                  const int (&col_lo)[NG], const int (&col_hi)[NG],
                                                  f32x4_t (&acc)[NG][2 * NQK], float (&m)[NG], f32x4_t (&negm)[NG],
-                                                 float (&l)[NG], const ScoreScale& scale) {
+                                                 float (&l)[NG], const ScoreScale& scale,
+                                                 const float* bias_row = nullptr, int bias_last = 0) {
   using S = PrefillStage<NQK>;
   const int lane = threadIdx.x & 63, g = lane >> 4, c = lane & 15;
   f32x4_t s[NG][2];
@@ -899,8 +939,8 @@ __device__ __forceinline__ void process_tile_lds(const unsigned char* __restrict
         s[q][sb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qreg[q][ch].v, ch == 0 ? negm[q] : s[q][sb], 0, 0, 0);
     }
   Pack8 p[NG];
-  prompt_tile_softmax<NQK, NG, masked>(s, key0, [g](int sb, int r) { return 16 * sb + 4 * g + r; }, col_lo, col_hi,
-                                       acc, m, negm, l, p, scale);
+  prompt_tile_softmax<NQK, NG, masked, EXTRA>(s, key0, [g](int sb, int r) { return 16 * sb + 4 * g + r; }, col_lo, col_hi,
+                                              acc, m, negm, l, p, scale, bias_row, bias_last);
 #pragma unroll
   for (int n = 0; n < 2 * NQK; ++n) {
     Pack8 vf;
@@ -915,14 +955,14 @@ __device__ __forceinline__ void process_tile_lds(const unsigned char* __restrict
 // their own and hand their (reference value, sum, output) to the lower four at the end.  A block then
 // lasts half as long and a compute unit holds one block at a time, so that blocks that finish early
 // (tiles with few keys) make room for the next ones instead of idling beside a long one.
-template <int NQK, int KS>
+template <int NQK, int KS, bool EXTRA = false>
 __global__ void __launch_bounds__(64 * PREFILL_WAVES * KS, NQK <= 4 ? 2 / KS : 1)
 attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
                          const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
                          const int* __restrict__ tiles, const int* __restrict__ positions,
                          const int* __restrict__ token_entry, const int* __restrict__ block_table,
                          int bt_stride, int page_size, int nq, int nkv, float scale_log2e, int window,
-                         int n_tiles) {
+                         int n_tiles, ScoreExtras extras) {
   using S = PrefillStage<NQK>;
   constexpr int HD = 32 * NQK;
   constexpr int NG = PREFILL_GROUPS;
@@ -948,6 +988,8 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
   const int head_in_group = (rest % chunks) * PREFILL_WAVES + wave;
   const bool head_ok = head_in_group < G;                 // a wave without a head still helps to load
   const int head = kvh * G + (head_ok ? head_in_group : G - 1);
+  const float* const bias_row = EXTRA && extras.bias ? extras.bias + (size_t)head * extras.bias_rows : nullptr;
+  const int bias_last = extras.bias_rows - 1;
   const int first = tiles[2 * tile_idx], count = tiles[2 * tile_idx + 1];
   int clo[NG], chi[NG], tok[NG];
   Pack8 qreg[NG][NQK];
@@ -1016,9 +1058,9 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
   do {                                                                             \
     const unsigned char* kl = tile_lds + (BUF) * TILE_BYTES;                       \
     if ((K0) + 31 > first_pos || (K0) < open_lo)                                   \
-      process_tile_lds<NQK, NG, true>(kl, kl + S::KBYTES, (K0), qreg, clo, chi, acc, m, negm, l, score_scale);  \
+      process_tile_lds<NQK, NG, true, EXTRA>(kl, kl + S::KBYTES, (K0), qreg, clo, chi, acc, m, negm, l, score_scale, bias_row, bias_last);  \
     else                                                                           \
-      process_tile_lds<NQK, NG, false>(kl, kl + S::KBYTES, (K0), qreg, clo, chi, acc, m, negm, l, score_scale); \
+      process_tile_lds<NQK, NG, false, EXTRA>(kl, kl + S::KBYTES, (K0), qreg, clo, chi, acc, m, negm, l, score_scale, bias_row, bias_last); \
     STAGE_STORE(NEXT, (K0) + 32, 1 - (BUF));                                       \
     STAGE_LOAD(NEXT, (K0) + 96);                                                   \
     __syncthreads();                                                               \
@@ -1032,9 +1074,9 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
   do {                                                                             \
     const unsigned char* kl = tile_lds + (BUF) * TILE_BYTES;                       \
     if ((K0) + 31 > first_pos || (K0) < open_lo)                                   \
-      process_tile_lds<NQK, NG, true>(kl, kl + S::KBYTES, (K0), qreg, clo, chi, acc, m, negm, l, score_scale);  \
+      process_tile_lds<NQK, NG, true, EXTRA>(kl, kl + S::KBYTES, (K0), qreg, clo, chi, acc, m, negm, l, score_scale, bias_row, bias_last);  \
     else                                                                           \
-      process_tile_lds<NQK, NG, false>(kl, kl + S::KBYTES, (K0), qreg, clo, chi, acc, m, negm, l, score_scale); \
+      process_tile_lds<NQK, NG, false, EXTRA>(kl, kl + S::KBYTES, (K0), qreg, clo, chi, acc, m, negm, l, score_scale, bias_row, bias_last); \
   } while (0)
   // Steps go in pairs, so that the two register stages and the two LDS tiles take turns in a way the
   // compiler can see (it then waits for the loads of two steps ago only); an odd last step follows the
@@ -1096,7 +1138,8 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
     lt += __shfl_xor(lt, 16, 64);
     lt += __shfl_xor(lt, 32, 64);
     if (chi[qg] < 0) continue;
-    const float inv = lt > 0.f ? 1.f / lt : 0.f;
+    float inv = lt > 0.f ? 1.f / lt : 0.f;
+    if constexpr (EXTRA) inv *= gate_of(extras, tok[qg], head);
     bf16_t* op = out + (size_t)tok[qg] * out_stride + (size_t)head * HD;
 #pragma unroll
     for (int n = 0; n < 2 * NQK; ++n)
@@ -1478,8 +1521,11 @@ static int decode_launch(
     const void* q, int q_stride, void* out, int out_stride, const void* k_pool, const void* v_pool,
     const int* token_list, int n_items, const int* positions, const int* token_entry,
     const int* block_table, int bt_stride, int page_size, int nq, int nkv, int hd, float scale, int window,
-    int num_splits, int waves, float* workspace, hipStream_t stream, const DecodeFuse* fuse = nullptr) {
+    int num_splits, int waves, float* workspace, hipStream_t stream, const DecodeFuse* fuse = nullptr,
+    const ScoreExtras* extras = nullptr) {
   if (n_items <= 0) return 0;
+  if (extras && fuse) return ULLM_ERR_UNSUPPORTED;
+  if (extras && extras->bias && extras->bias_rows <= 0) return ULLM_ERR_SHAPE;
   if (!ullm_attention_mfma_supports(hd, page_size, nq, nkv)) return ULLM_ERR_UNSUPPORTED;
   if (waves != 1 && waves != 4 && waves != 8) return ULLM_ERR_UNSUPPORTED;
   if (hd == 256 && waves == 8) waves = 4;                // shared memory of the merge
@@ -1491,13 +1537,21 @@ static int decode_launch(
   dim3 grid(num_splits, nkv * groups, n_items), block(64 * waves);
   const DecodeFuse f = fuse ? *fuse : DecodeFuse{nullptr, nullptr, 0.f, nullptr, 0, nullptr, nullptr};
 #define ARGS (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, token_list, \
-    positions, token_entry, block_table, bt_stride, page_size, nq, nkv, sl, window, num_splits, workspace, f
+    positions, token_entry, block_table, bt_stride, page_size, nq, nkv, sl, window, num_splits, workspace, f, x
+  const ScoreExtras x = extras ? *extras : ScoreExtras{nullptr, 0, nullptr, 0};
 #define CALL_AS(N, F) do {                                                                                     \
     if (waves == 8) hipLaunchKernelGGL((attention_decode_kernel<N, 8, F>), grid, block, 0, stream, ARGS);      \
     else if (waves == 4) hipLaunchKernelGGL((attention_decode_kernel<N, 4, F>), grid, block, 0, stream, ARGS); \
     else hipLaunchKernelGGL((attention_decode_kernel<N, 1, F>), grid, block, 0, stream, ARGS);                 \
   } while (0)
-  if (fuse) {
+#define CALL_EXTRA(N) do {                                                                                               \
+    if (waves == 8) hipLaunchKernelGGL((attention_decode_kernel<N, 8, false, true>), grid, block, 0, stream, ARGS);      \
+    else if (waves == 4) hipLaunchKernelGGL((attention_decode_kernel<N, 4, false, true>), grid, block, 0, stream, ARGS); \
+    else hipLaunchKernelGGL((attention_decode_kernel<N, 1, false, true>), grid, block, 0, stream, ARGS);                 \
+  } while (0)
+  if (extras) {
+    DISPATCH_NQK(hd, CALL_EXTRA)
+  } else if (fuse) {
     switch (hd) {
       case 64: CALL_AS(2, true); break;
       case 128: CALL_AS(4, true); break;
@@ -1510,12 +1564,27 @@ static int decode_launch(
 #undef CALL
   }
 #undef CALL_AS
+#undef CALL_EXTRA
 #undef ARGS
   int rc = (int)hipGetLastError();
   if (rc != 0 || num_splits == 1) return rc;
   hipLaunchKernelGGL(attention_reduce_kernel, dim3(n_items, nq), dim3(64), 0, stream, workspace, (bf16_t*)out,
-                     out_stride, token_list, nq, hd, num_splits);
+                     out_stride, token_list, nq, hd, num_splits, x);
   ULLM_LAUNCH_CHECK();
+}
+
+// ullm_attention_decode with a bias by distance on the scores (float32 [nq][bias_rows], already multiplied by
+// log2(e); null for none) and a gate per head on the outputs (bfloat16 [tokens][gate_stride]; null for none).
+extern "C" int ullm_attention_decode_extras(
+    const void* q, int q_stride, void* out, int out_stride, const void* k_pool, const void* v_pool,
+    const int* token_list, int n_items, const int* positions, const int* token_entry,
+    const int* block_table, int bt_stride, int page_size, int nq, int nkv, int hd, float scale, int window,
+    int num_splits, int waves, float* workspace, const float* bias, int bias_rows, const void* gate, int gate_stride,
+    hipStream_t stream) {
+  const ScoreExtras x{bias, bias_rows, (const bf16_t*)gate, gate_stride};
+  return decode_launch(q, q_stride, out, out_stride, k_pool, v_pool, token_list, n_items, positions, token_entry,
+                       block_table, bt_stride, page_size, nq, nkv, hd, scale, window, num_splits, waves, workspace,
+                       stream, nullptr, &x);
 }
 
 extern "C" int ullm_attention_decode(
@@ -1612,7 +1681,19 @@ extern "C" int ullm_attention_decode_static(
 }
 
 template <int N, typename... Args>
+static void prefill_launch_extras(int halves, unsigned blocks, hipStream_t stream, Args... args) {
+  if constexpr (N <= 4) {
+    if (halves == 2) {
+      hipLaunchKernelGGL((attention_prefill_kernel<N, 2, true>), dim3(blocks), dim3(64 * PREFILL_WAVES * 2), 0, stream, args...);
+      return;
+    }
+  }
+  hipLaunchKernelGGL((attention_prefill_kernel<N, 1, true>), dim3(blocks), dim3(64 * PREFILL_WAVES), 0, stream, args...);
+}
+
+template <int N, typename... Args>
 static void prefill_launch(int halves, bool staged, unsigned blocks, hipStream_t stream, Args... args) {
+  const ScoreExtras none{nullptr, 0, nullptr, 0};
   if constexpr (N == 4) {
     if (!staged) {                                        // tiles straight to shared memory
       if (halves == 2)
@@ -1624,11 +1705,11 @@ static void prefill_launch(int halves, bool staged, unsigned blocks, hipStream_t
   }
   if constexpr (N <= 4) {
     if (halves == 2) {
-      hipLaunchKernelGGL((attention_prefill_kernel<N, 2>), dim3(blocks), dim3(64 * PREFILL_WAVES * 2), 0, stream, args...);
+      hipLaunchKernelGGL((attention_prefill_kernel<N, 2>), dim3(blocks), dim3(64 * PREFILL_WAVES * 2), 0, stream, args..., none);
       return;
     }
   }
-  hipLaunchKernelGGL((attention_prefill_kernel<N, 1>), dim3(blocks), dim3(64 * PREFILL_WAVES), 0, stream, args...);
+  hipLaunchKernelGGL((attention_prefill_kernel<N, 1>), dim3(blocks), dim3(64 * PREFILL_WAVES), 0, stream, args..., none);
 }
 
 // Compute units of the current device (asked once per device).
@@ -1651,12 +1732,13 @@ static int compute_units() {
 // keep every unit busy to the end); 0 = choose.  The choice compares the work per unit,
 // `keys_total` (sum over the tiles of the keys each sees) spread over two blocks per unit, with the
 // longest tile `keys_max`; without these figures (0) it goes by the number of blocks.
-extern "C" int ullm_attention_prefill(
+static int prefill_any(
     const void* q, int q_stride, void* out, int out_stride, const void* k_pool, const void* v_pool,
     const int* tiles, int n_tiles, const int* positions, const int* token_entry, const int* block_table,
     int bt_stride, int page_size, int nq, int nkv, int hd, float scale, int window, int halves,
-    long long keys_total, int keys_max, hipStream_t stream) {
+    long long keys_total, int keys_max, hipStream_t stream, const ScoreExtras* extras) {
   if (n_tiles <= 0) return 0;
+  if (extras && extras->bias && extras->bias_rows <= 0) return ULLM_ERR_SHAPE;
   if (!ullm_attention_mfma_supports(hd, page_size, nq, nkv)) return ULLM_ERR_UNSUPPORTED;
   const bool staged = halves >= 10;                       // 10, 11, 12: as 0, 1, 2 with the kernel that stages tiles in registers
   if (staged) halves -= 10;
@@ -1684,7 +1766,37 @@ extern "C" int ullm_attention_prefill(
 #define CALL(N) prefill_launch<N>(halves, staged, (unsigned)blocks, stream, (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, \
     (const bf16_t*)k_pool, (const bf16_t*)v_pool, tiles, positions, token_entry, block_table, bt_stride, page_size,    \
     nq, nkv, sl, window, n_tiles)
-  DISPATCH_NQK(hd, CALL)
+#define CALL_EXTRA(N) prefill_launch_extras<N>(halves, (unsigned)blocks, stream, (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, \
+    (const bf16_t*)k_pool, (const bf16_t*)v_pool, tiles, positions, token_entry, block_table, bt_stride, page_size,    \
+    nq, nkv, sl, window, n_tiles, *extras)
+  if (extras) {
+    DISPATCH_NQK(hd, CALL_EXTRA)
+  } else {
+    DISPATCH_NQK(hd, CALL)
+  }
 #undef CALL
+#undef CALL_EXTRA
   ULLM_LAUNCH_CHECK();
+}
+
+extern "C" int ullm_attention_prefill(
+    const void* q, int q_stride, void* out, int out_stride, const void* k_pool, const void* v_pool,
+    const int* tiles, int n_tiles, const int* positions, const int* token_entry, const int* block_table,
+    int bt_stride, int page_size, int nq, int nkv, int hd, float scale, int window, int halves,
+    long long keys_total, int keys_max, hipStream_t stream) {
+  return prefill_any(q, q_stride, out, out_stride, k_pool, v_pool, tiles, n_tiles, positions, token_entry, block_table,
+                     bt_stride, page_size, nq, nkv, hd, scale, window, halves, keys_total, keys_max, stream, nullptr);
+}
+
+// ullm_attention_prefill with a bias by distance on the scores and a gate per head on the outputs (as
+// ullm_attention_decode_extras); always the kernel that stages its tiles through registers.
+extern "C" int ullm_attention_prefill_extras(
+    const void* q, int q_stride, void* out, int out_stride, const void* k_pool, const void* v_pool,
+    const int* tiles, int n_tiles, const int* positions, const int* token_entry, const int* block_table,
+    int bt_stride, int page_size, int nq, int nkv, int hd, float scale, int window, int halves,
+    long long keys_total, int keys_max, const float* bias, int bias_rows, const void* gate, int gate_stride,
+    hipStream_t stream) {
+  const ScoreExtras x{bias, bias_rows, (const bf16_t*)gate, gate_stride};
+  return prefill_any(q, q_stride, out, out_stride, k_pool, v_pool, tiles, n_tiles, positions, token_entry, block_table,
+                     bt_stride, page_size, nq, nkv, hd, scale, window, halves % 10, keys_total, keys_max, stream, &x);
 }

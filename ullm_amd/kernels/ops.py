@@ -466,6 +466,12 @@ def gated_group_norm(y: torch.Tensor, proj: torch.Tensor, z_off: int, gain: torc
 
 # ---------------------------------------------------------------------------------- attention
 
+def _check_gate(gate: Optional[torch.Tensor], T: int, nq: int) -> None:
+    if gate is not None:
+        _need(gate.dtype == torch.bfloat16 and gate.dim() == 2 and gate.shape[0] == T and gate.shape[1] >= nq
+              and gate.stride(1) == 1, f"a head gate must be bfloat16 [T, >= {nq}]")
+
+
 def _check_distance_bias(bias: Optional[torch.Tensor], nq: int) -> int:
     """Rows of a distance-bias table (0 for none) after checking that it is float32 [nq, rows]."""
     if bias is None:
@@ -809,10 +815,12 @@ def decode_split(n_items: int, nkv: int, groups: int, max_kv: int, hd: int = 128
 
 def attention_decode_mfma(q, out, k_pool, v_pool, token_list: Optional[torch.Tensor], n_items: int,
                           positions, token_entry, block_table, page_size: int, nq: int, nkv: int, hd: int,
-                          scale: float, window: int, max_kv: int, splits: int = 0, waves: int = 0) -> None:
+                          scale: float, window: int, max_kv: int, splits: int = 0, waves: int = 0,
+                          bias_log2: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None) -> None:
     """One query token per item (``token_list`` int32 [n_items] names the tokens, None = tokens
     0..n_items-1) against its request's cache; with ``splits`` > 1 the keys go to several blocks whose
-    partial results a second small kernel adds up."""
+    partial results a second small kernel adds up.  ``bias_log2`` (float32 [nq, rows], a distance bias times
+    log2(e)) is added to the scores, ``gate`` (bfloat16 [T, >= nq]) gates every head's output by its sigmoid."""
     _check_pools(k_pool, v_pool, nkv, page_size, hd, torch.bfloat16)
     _need(q.dtype == torch.bfloat16 and q.stride(1) == 1 and q.shape[1] == nq * hd, "q must be bfloat16 [T, nq*hd]")
     _need(out.dtype == torch.bfloat16 and out.stride(1) == 1 and out.shape == q.shape, "bad attention output")
@@ -835,6 +843,15 @@ def attention_decode_mfma(q, out, k_pool, v_pool, token_list: Optional[torch.Ten
     ws = None
     if splits > 1:
         ws = torch.empty(n_items * nq * splits * (hd + 4), dtype=torch.float32, device=q.device)
+    if bias_log2 is not None or gate is not None:
+        _check_gate(gate, q.shape[0], nq)
+        _check(lib.ullm_attention_decode_extras(
+            _p(q), _c_int(q.stride(0)), _p(out), _c_int(out.stride(0)), _p(k_pool), _p(v_pool), _p(token_list),
+            _c_int(n_items), _p(positions), _p(token_entry), _p(block_table), _c_int(block_table.stride(0)),
+            _c_int(page_size), _c_int(nq), _c_int(nkv), _c_int(hd), _c_float(scale), _c_int(window),
+            _c_int(splits), _c_int(waves), _p(ws), _p(bias_log2), _c_int(_check_distance_bias(bias_log2, nq)), _p(gate),
+            _c_int(gate.stride(0) if gate is not None else 0), _stream()), "attention_decode_extras")
+        return
     _check(lib.ullm_attention_decode(
         _p(q), _c_int(q.stride(0)), _p(out), _c_int(out.stride(0)), _p(k_pool), _p(v_pool), _p(token_list),
         _c_int(n_items), _p(positions), _p(token_entry), _p(block_table), _c_int(block_table.stride(0)),
@@ -906,7 +923,8 @@ PREFILL_TILE = 32      # tokens of one request per prompt tile (two groups of 16
 
 def attention_prefill_mfma(q, out, k_pool, v_pool, tiles: torch.Tensor, n_tiles: int, positions, token_entry,
                            block_table, page_size: int, nq: int, nkv: int, hd: int, scale: float,
-                           window: int, halves: int = 0, keys_total: int = 0, keys_max: int = 0) -> None:
+                           window: int, halves: int = 0, keys_total: int = 0, keys_max: int = 0,
+                           bias_log2: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None) -> None:
     """Tiles (first token, count <= PREFILL_TILE) of consecutive tokens of one request each, every
     token against the keys up to its own position.  ``halves``: 2 = two halves of a block share a
     tile's keys, 1 = one block takes them all, 0 = chosen from ``keys_total`` (the sum over the tiles of
@@ -921,6 +939,16 @@ def attention_prefill_mfma(q, out, k_pool, v_pool, tiles: torch.Tensor, n_tiles:
     _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.stride(1) == 1,
           "block_table must be int32 [B, stride]")
     lib = build.load("attention_mfma")
+    if bias_log2 is not None or gate is not None:
+        _check_gate(gate, q.shape[0], nq)
+        _check(lib.ullm_attention_prefill_extras(
+            _p(q), _c_int(q.stride(0)), _p(out), _c_int(out.stride(0)), _p(k_pool), _p(v_pool), _p(tiles),
+            _c_int(n_tiles), _p(positions), _p(token_entry), _p(block_table), _c_int(block_table.stride(0)),
+            _c_int(page_size), _c_int(nq), _c_int(nkv), _c_int(hd), _c_float(scale), _c_int(window),
+            _c_int(halves), ctypes.c_longlong(int(keys_total)), _c_int(keys_max), _p(bias_log2),
+            _c_int(_check_distance_bias(bias_log2, nq)), _p(gate), _c_int(gate.stride(0) if gate is not None else 0),
+            _stream()), "attention_prefill_extras")
+        return
     _check(lib.ullm_attention_prefill(
         _p(q), _c_int(q.stride(0)), _p(out), _c_int(out.stride(0)), _p(k_pool), _p(v_pool), _p(tiles),
         _c_int(n_tiles), _p(positions), _p(token_entry), _p(block_table), _c_int(block_table.stride(0)),
@@ -949,29 +977,36 @@ def _warn_general_attention(hd: int, page_size: int) -> None:
 
 def paged_attention(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, ctx, group, nq: int,
                     nkv: int, hd: int, scale: float, window: int, plan=None,
-                    bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+                    bias: Optional[torch.Tensor] = None, bias_log2: Optional[torch.Tensor] = None,
+                    gate: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention of the batch's queries over their requests' cached keys and values (the new
     tokens' rows included).  bfloat16 shapes the matrix-core kernels take go there (one launch for
     the one-token entries, one for the tiles of longer entries, both listed in ``plan``: arrays
     ``decode_tokens`` and ``tiles``, numbers ``num_decode``, ``max_decode_kv``, ``num_tiles``,
     ``tile_keys_total``, ``tile_keys_max``); everything else, and float32 always, takes the general
-    kernel.  Every choice computes the same function."""
-    if bias is not None or not attention_mfma_supports(q.dtype, hd, group.page_size, nq, nkv):
-        if q.dtype == torch.bfloat16 and bias is None:
+    kernel.  Every choice computes the same function.  ``bias`` (float32 [nq, rows]) is a bias by distance on the
+    scores (``bias_log2``: the same times log2(e), which the matrix-core kernels add to their exponents of two);
+    ``gate`` [T, >= nq]: every head's output is multiplied by the sigmoid of its gate."""
+    if not attention_mfma_supports(q.dtype, hd, group.page_size, nq, nkv):
+        if q.dtype == torch.bfloat16:
             _warn_general_attention(hd, group.page_size)
-        return paged_attention_generic(q, k_pool, v_pool, ctx.positions, ctx.token_entry, group.block_table,
-                                       group.page_size, nq, nkv, hd, scale, window, bias=bias)
+        out = paged_attention_generic(q, k_pool, v_pool, ctx.positions, ctx.token_entry, group.block_table,
+                                      group.page_size, nq, nkv, hd, scale, window, bias=bias)
+        return out if gate is None else head_gate_(out, gate, nq, hd)
+    if bias is not None:
+        _need(bias_log2 is not None and bias_log2.shape == bias.shape, "the matrix-core kernels take the bias times log2(e)")
     _need(plan is not None, "the matrix-core attention kernels need the step's work lists (a step plan)")
     out = torch.empty((q.shape[0], nq * hd), dtype=q.dtype, device=q.device)
     n = plan.facts
     if n["num_decode"]:
         attention_decode_mfma(q, out, k_pool, v_pool, plan.arrays["decode_tokens"], n["num_decode"], ctx.positions,
                               ctx.token_entry, group.block_table, group.page_size, nq, nkv, hd, scale, window,
-                              n["max_decode_kv"])
+                              n["max_decode_kv"], bias_log2=bias_log2 if bias is not None else None, gate=gate)
     if n["num_tiles"]:
         attention_prefill_mfma(q, out, k_pool, v_pool, plan.arrays["tiles"], n["num_tiles"], ctx.positions,
                                ctx.token_entry, group.block_table, group.page_size, nq, nkv, hd, scale, window,
-                               keys_total=n["tile_keys_total"], keys_max=n["tile_keys_max"])
+                               keys_total=n["tile_keys_total"], keys_max=n["tile_keys_max"],
+                               bias_log2=bias_log2 if bias is not None else None, gate=gate)
     return out
 
 

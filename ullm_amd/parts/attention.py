@@ -268,9 +268,10 @@ class GQAttention(Mixer):
                                     self.qk_norm_eps or 0.0, nq * self.dim, nkv * self.dim, ctx.positions,
                                     ctx.token_entry, group.block_table, cache.k_pool, cache.v_pool, group.page_size,
                                     nq, nkv, hd, has_kv=self.own_kv)
+        bias = self.position.score_bias() if self.position is not None else None
+        # the bias joins the scores and the gate the heads' outputs inside the attention kernels
         out = ops.paged_attention(q, cache.k_pool, cache.v_pool, ctx, group, nq, nkv, hd, self.scale, self.window,
-                                  ctx.plans["attention"],
-                                  bias=self.position.score_bias() if self.position is not None else None)
-        if self.head_gate:
-            ops.head_gate_(out, proj[:, self.gate_off:], nq, hd)
+                                  ctx.plans["attention"], bias=bias,
+                                  bias_log2=self.position.score_bias_log2() if bias is not None else None,
+                                  gate=proj[:, self.gate_off:] if self.head_gate else None)
         return linear_into_stream(out, self.w_o, ctx)

@@ -104,6 +104,11 @@ class LogDistanceBias(PositionEncoding):
                              f"two rows and a reach beyond rows // 2")
         index = torch.tensor(self.buckets(), dtype=torch.long, device=table.device)
         self.by_distance = table[index].T.contiguous()           # [heads, distances]
+        self.by_distance_log2 = (self.by_distance * math.log2(math.e)).contiguous()
 
     def score_bias(self):
         return self.by_distance
+
+    def score_bias_log2(self):
+        """The same table times log2(e), for kernels whose scores are exponents of two."""
+        return self.by_distance_log2
