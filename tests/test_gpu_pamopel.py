@@ -355,3 +355,49 @@ def test_the_trace_program_runs_the_design(models, trace_run):
     b = tr.step([("a", toks[21:], [18])], end=["a"])
     tr.close()
     close(np.concatenate((a, b)), want[[0, 20, 39]], "float32")
+
+
+@pytest.mark.parametrize("hd,nq,nkv", [(64, 8, 1), (128, 6, 2), (32, 20, 1), (96, 4, 4), (256, 2, 1)])
+def test_matrix_core_attention_with_distance_bias_and_head_gates(hd, nq, nkv):
+    """The bfloat16 kernels (single tokens cut over splits and their reduce; prompt tiles) against 64-bit softmax
+    attention on the same rounded operands: a bias by distance whose entries are units apart, clamped at the
+    table's last entry, and a gate per head; contexts that end at and beside tile and page borders, one past 1 100
+    keys; a prompt portion that starts in the middle of a page beside single tokens."""
+    import math
+    from types import SimpleNamespace
+    from gpu_util import paged_cache, table_tensor
+    from ullm_amd.kernels import ops
+    from ullm_amd.parts import GroupView, StepShape
+    from ullm_amd.parts.attention import plan_attention_step
+    g = torch.Generator().manual_seed(hd + nq)
+    starts, lens = [1130, 31, 64, 200, 0], [1, 1, 1, 45, 33]            # tokens before the step, new tokens
+    rows = 70
+    bias = (torch.randn(nq, rows, generator=g) * 2).float()
+    seqs_k = [torch.randn(s + n, nkv, hd, generator=g).bfloat16().float() for s, n in zip(starts, lens)]
+    seqs_v = [torch.randn(s + n, nkv, hd, generator=g).bfloat16().float() for s, n in zip(starts, lens)]
+    k_pool, v_pool, tables = paged_cache(seqs_k, seqs_v, 16, torch.bfloat16, DEV, fill=0.0)
+    T = sum(lens)
+    q = torch.randn(T, nq, hd, generator=g).bfloat16()
+    gate = torch.randn(T, nq + 3, generator=g).bfloat16()
+    positions = torch.tensor([s + i for s, n in zip(starts, lens) for i in range(n)], dtype=torch.int32, device=DEV)
+    entry = torch.tensor([b for b, n in enumerate(lens) for _ in range(n)], dtype=torch.int32, device=DEV)
+    plan = plan_attention_step(StepShape(tuple(lens), tuple(starts)))
+    plan.arrays = {k: torch.tensor(v, dtype=torch.int32, device=DEV) for k, v in plan.arrays.items()}
+    group = GroupView(table_tensor(tables, DEV), 0, 16, 0)
+    ctx = SimpleNamespace(positions=positions, token_entry=entry)
+    scale = 0.7 / math.sqrt(hd)
+    out = ops.paged_attention(q.view(T, nq * hd).to(DEV), k_pool, v_pool, ctx, group, nq, nkv, hd, scale, 0, plan,
+                              bias=bias.to(DEV), bias_log2=(bias * math.log2(math.e)).to(DEV), gate=gate.to(DEV))
+    out = out.float().cpu().view(T, nq, hd)
+    t = 0
+    for b, (s, n) in enumerate(zip(starts, lens)):
+        for i in range(n):
+            pos = s + i
+            dist = (pos - torch.arange(pos + 1)).clamp(max=rows - 1)
+            for h in range(nq):
+                kv = h // (nq // nkv)
+                sc = (seqs_k[b][:pos + 1, kv].double() @ q[t, h].double()) * scale + bias[h][dist].double()
+                want = (torch.softmax(sc, 0) @ seqs_v[b][:pos + 1, kv].double()) * torch.sigmoid(gate[t, h].double())
+                err = (out[t, h].double() - want).abs().max()
+                assert err <= 2e-2 * max(1.0, float(want.abs().max())), (b, i, h, float(err))
+            t += 1
