@@ -51,6 +51,12 @@ def parse_args():
     ap.add_argument("--mixed-only", action="store_true",
                     help="only the reference's own workload: 256 requests of mixed lengths "
                          "(Qwen3-0.6B sizes unless --size is given)")
+    ap.add_argument("--design", choices=sorted(DESIGN_SHAPES), default=None, metavar="SHAPE",
+                    help="instead of the default workload: Pamopel (attention with a distance bias and head gates, a "
+                         "layer on another's keys and values, a Mamba-2 layer) beside a Qwen3 stack of the same width, "
+                         f"heads, feed-forward, vocabulary and depth, random weights; shapes: {sorted(DESIGN_SHAPES)}")
+    ap.add_argument("--design-model", choices=("both", "pamopel", "qwen3"), default="both",
+                    help="with --design: run one of the two designs only (for profiles)")
     ap.add_argument("--prefill-only", type=int, default=0, metavar="T",
                     help="only time a T-token prompt and print its figures (for profiling)")
     return ap.parse_args()
@@ -119,20 +125,72 @@ def measured_peaks():
     return {"read_GBs": round(read_gbs, 1), "copy_GBs": round(copy_gbs, 1), "gemm_bf16_8192_TFLOPs": round(gemm_tflops, 1)}
 
 
+# Layer shapes for --design: (width, query heads, kv heads, head size, feed-forward, layers) and the
+# state-space layer's (heads, head size, state, groups).  Vocabulary 32 768 for both designs.
+DESIGN_SHAPES = {"2048": ((2048, 16, 8, 128, 6144, 8), (64, 64, 128, 8)),
+                 "4096": ((4096, 32, 8, 128, 12288, 8), (128, 64, 128, 8))}
+DESIGN_VOCAB = 32768
+
+
+def design_configs(shape):
+    """(Pamopel config.json, Qwen3 config.json) of one shape: Pamopel's layers repeat attention, attention on the
+    layer before's keys and values, Mamba-2, attention; every layer has the feed-forward."""
+    (W, H, G, D, F, L), (mh, mp, mn, mg) = DESIGN_SHAPES[shape]
+    att = dict(heads=H, kv_heads=G, dim=D, vdim=D, scale=D ** -0.5, bias_max=1024)
+    mlp = dict(kind="dense", ff=F)
+    layers = []
+    for i in range(L):
+        kind = i % 4
+        if kind == 2:
+            layers.append(dict(type="mamba2", mlp=mlp, mixer=dict(heads=mh, vdim=mp, state=mn, groups=mg, conv=4, norm_groups=mg)))
+        else:
+            layers.append(dict(type="attention", mlp=mlp, mixer=dict(att, kv_from=i - 1) if kind == 1 else dict(att)))
+    pamopel = dict(architecture="Pamopel", vocab=DESIGN_VOCAB, width=W, layers=layers, norm=dict(eps=1e-5), residual_mult=0.5,
+                   logit_scale=1.0, embedding=dict(scale=1.0, bigram=dict(buckets=65521, mul_prev=31, mul_cur=17)))
+    qwen = dict(architectures=["Qwen3ForCausalLM"], hidden_size=W, num_hidden_layers=L, num_attention_heads=H,
+                num_key_value_heads=G, head_dim=D, intermediate_size=F, vocab_size=DESIGN_VOCAB, rope_theta=1e6,
+                rms_norm_eps=1e-6, max_position_embeddings=40960, tie_word_embeddings=False, attention_bias=False,
+                use_sliding_window=False, initializer_range=0.02, torch_dtype="bfloat16")
+    return pamopel, qwen
+
+
+def design_run(args):
+    """Decode at batch 1 / 8 / 64 (1024-token prompts) and one 2048-token prompt, for both designs of a shape."""
+    out = {"metric": f"decode and prefill tok/s, Pamopel beside Qwen3 at shape {args.design}, random weights",
+           "unit": "tokens/s", "dtype": args.dtype, "data": "synthetic", "shape": args.design, "designs": {}}
+    for label, config in zip(("pamopel", "qwen3"), design_configs(args.design)):
+        if args.design_model not in ("both", label):
+            continue
+        m = Sized(label, args.dtype, 4096, eager=args.eager, config=config)
+        rec = {"weights_GB": round(m.wbytes / 1e9, 3), "decode": {}}
+        for batch in (1, 8, 64):
+            tok_s, ms, _, ctx = m.decode(batch, args.steps, args.warmup, 1024)
+            rec["decode"][f"b{batch}"] = {"tok_s": round(tok_s, 1), "ms_per_step": round(ms, 3), "context": round(ctx)}
+        p_tok_s, p_ms, _ = m.prefill(2048)
+        rec["prefill_2048"] = {"tok_s": round(p_tok_s, 1), "ms": round(p_ms, 3)}
+        out["designs"][label] = rec
+        m.close()
+    print(json.dumps(out))
+    return 0
+
+
 class Sized:
     """A model of one named size with random weights on the device, and the runs it is timed on."""
 
-    def __init__(self, size, dtype, context_len, layers=None, eager=False, longest_context=None):
+    def __init__(self, size, dtype, context_len, layers=None, eager=False, longest_context=None, config=None):
+        """``config``: a config.json dict of any registered architecture instead of a named Qwen3 size
+        (``size`` is then only its label)."""
         import torch
         from ullm_amd.config import parse_random_weights
         from ullm_amd.engine.loading import make_env
         from ullm_amd.models import build_model
         from ullm_amd.weights.random_init import bind_random_weights
         self.torch, self.size, self.dtype, self.context_len, self.eager = torch, size, dtype, context_len, eager
-        config, _ = parse_random_weights(f"qwen3-{size}")
-        self.full_layers = config["num_hidden_layers"]
-        if layers is not None:
-            config["num_hidden_layers"] = layers
+        if config is None:
+            config, _ = parse_random_weights(f"qwen3-{size}")
+            self.full_layers = config["num_hidden_layers"]
+            if layers is not None:
+                config["num_hidden_layers"] = layers
         self.cfg, self.model = build_model(config)
         # the model (its position table) is built once for the longest context any point runs at; every engine
         # gets an environment with its own context length (block tables as wide as that context needs)
@@ -222,6 +280,8 @@ class Sized:
                 best = dt if best is None else min(best, dt)
         del eng
         torch.cuda.empty_cache()
+        if not hasattr(self.cfg, "num_attention_heads"):
+            return n_tokens / best, best * 1e3, None        # no flop count for this architecture
         flops = step_flops(self.cfg, n_tokens, n_tokens * (n_tokens + 1) // 2, 1)
         return n_tokens / best, best * 1e3, flops / best / PEAK_FLOPS[self.dtype]
 
@@ -273,6 +333,8 @@ def main():
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+    if args.design:
+        return design_run(args)
     if args.mixed_only:
         size = args.size or "0.6b"
         m = Sized(size, args.dtype, 4096, eager=args.eager)

@@ -923,6 +923,92 @@ add_norm_general_kernel(const TB* __restrict__ branch, float* __restrict__ resid
   for (int c = threadIdx.x; c < H; c += blockDim.x) st_f32(out + c, ((row[c] - mean) * rs) * gain[c]);
 }
 
+// Two block sums with one pair of barriers.
+__device__ __forceinline__ void block_sum2(float& a, float& b, float* scratch /* 32 floats */) {
+  const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+  const int nwaves = (blockDim.x + WAVE - 1) / WAVE;
+  a = wave_sum(a);
+  b = wave_sum(b);
+  __syncthreads();
+  if (lane == 0) {
+    scratch[wave] = a;
+    scratch[16 + wave] = b;
+  }
+  __syncthreads();
+  float ra = 0.f, rb = 0.f;
+  for (int w = 0; w < nwaves; ++w) {
+    ra += scratch[w];
+    rb += scratch[16 + w];
+  }
+  a = ra;
+  b = rb;
+}
+
+// The same function for rows of up to 256 * K values, held in registers: every operand a thread needs (branch,
+// stream, both gains) is asked for before the first sum, so the row costs one trip to memory and four block sums.
+template <typename TB, typename TY, int K>
+__global__ void __launch_bounds__(256)
+add_norm_general_reg_kernel(const TB* __restrict__ branch, float* __restrict__ residual,
+                            const float* __restrict__ post_gain, float post_eps, int post_kind, float mult,
+                            const float* __restrict__ gain, float eps, int kind, TY* __restrict__ y,
+                            const int* __restrict__ rows, int H, int write_res) {
+  __shared__ float scratch[16];
+  const int r = blockIdx.x;
+  const int i = rows ? rows[r] : r;
+  float* res = residual + (size_t)i * H;
+  const float inv_h = 1.f / (float)H;
+  float v[K], s[K], pg[K], gn[K];
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    const int c = threadIdx.x + 256 * k;
+    const bool in = c < H;
+    const int cc = in ? c : H - 1;
+    s[k] = res[cc];
+    v[k] = branch ? ld_f32(branch + (size_t)i * H + cc) : 0.f;
+    pg[k] = post_gain ? post_gain[cc] : 1.f;
+    gn[k] = y ? gain[cc] : 1.f;
+    if (!in) { s[k] = 0.f; v[k] = 0.f; }
+  }
+  if (branch) {
+    if (post_gain) {
+      float sum = 0.f;
+#pragma unroll
+      for (int k = 0; k < K; ++k) sum += v[k];
+      const float mean = post_kind == 1 ? block_sum(sum, scratch) * inv_h : 0.f;
+      float ss = 0.f;
+#pragma unroll
+      for (int k = 0; k < K; ++k) {
+        const float d = threadIdx.x + 256 * k < H ? v[k] - mean : 0.f;
+        ss += d * d;
+      }
+      const float rs = 1.f / sqrtf(block_sum(ss, scratch) * inv_h + post_eps);
+#pragma unroll
+      for (int k = 0; k < K; ++k) v[k] = ((v[k] - mean) * rs) * pg[k];
+    }
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      s[k] = s[k] + mult * v[k];
+      if (write_res && threadIdx.x + 256 * k < H) res[threadIdx.x + 256 * k] = s[k];
+    }
+  }
+  if (!y) return;
+  float sum = 0.f;
+#pragma unroll
+  for (int k = 0; k < K; ++k) sum += threadIdx.x + 256 * k < H ? s[k] : 0.f;
+  const float mean = kind == 1 ? block_sum(sum, scratch) * inv_h : 0.f;
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    const float d = threadIdx.x + 256 * k < H ? s[k] - mean : 0.f;
+    ss += d * d;
+  }
+  const float rs = 1.f / sqrtf(block_sum(ss, scratch) * inv_h + eps);
+  TY* out = y + (size_t)r * H;
+#pragma unroll
+  for (int k = 0; k < K; ++k)
+    if (threadIdx.x + 256 * k < H) st_f32(out + threadIdx.x + 256 * k, ((s[k] - mean) * rs) * gn[k]);
+}
+
 extern "C" int ullm_add_norm_general(const void* branch, float* residual, const float* post_gain, float post_eps,
                                      int post_kind, float mult, const float* gain, float eps, int kind, void* y,
                                      const int* rows, int n_rows, int H, int branch_dtype, int y_dtype, int write_res,
@@ -931,14 +1017,23 @@ extern "C" int ullm_add_norm_general(const void* branch, float* residual, const 
   if (H <= 0 || H > 16384 || (kind != 0 && kind != 1) || (post_kind != 0 && post_kind != 1) || (y && !gain))
     return ULLM_ERR_SHAPE;
   const size_t shared = (size_t)H * sizeof(float);
-#define GO(TB, TY) hipLaunchKernelGGL((add_norm_general_kernel<TB, TY>), dim3(n_rows), dim3(256), shared, stream, \
+#define GO_K(TB, TY, K) hipLaunchKernelGGL((add_norm_general_reg_kernel<TB, TY, K>), dim3(n_rows), dim3(256), 0, stream, \
     (const TB*)branch, residual, post_gain, post_eps, post_kind, mult, gain, eps, kind, (TY*)y, rows, H, write_res)
+#define GO(TB, TY) do {                                                                                              \
+    if (H <= 512) GO_K(TB, TY, 2);                                                                                   \
+    else if (H <= 1024) GO_K(TB, TY, 4);                                                                             \
+    else if (H <= 2048) GO_K(TB, TY, 8);                                                                             \
+    else if (H <= 4096) GO_K(TB, TY, 16);                                                                            \
+    else hipLaunchKernelGGL((add_norm_general_kernel<TB, TY>), dim3(n_rows), dim3(256), shared, stream,             \
+    (const TB*)branch, residual, post_gain, post_eps, post_kind, mult, gain, eps, kind, (TY*)y, rows, H, write_res); \
+  } while (0)
   if (branch_dtype == ULLM_F32 && y_dtype == ULLM_F32) GO(float, float);
   else if (branch_dtype == ULLM_BF16 && y_dtype == ULLM_BF16) GO(bf16_t, bf16_t);
   else if (branch_dtype == ULLM_F32 && y_dtype == ULLM_BF16) GO(float, bf16_t);
   else if (branch_dtype == ULLM_BF16 && y_dtype == ULLM_F32) GO(bf16_t, float);
   else return ULLM_ERR_DTYPE;
 #undef GO
+#undef GO_K
   ULLM_LAUNCH_CHECK();
 }
 
@@ -957,39 +1052,40 @@ qk_whole_norm_write_kernel(const T* __restrict__ proj, int proj_stride, int q_of
                            const int* __restrict__ positions, const int* __restrict__ token_entry,
                            const int* __restrict__ block_table, int bt_stride, T* __restrict__ k_pool,
                            T* __restrict__ v_pool, int page_size, int nq, int nkv, int hd, int has_kv) {
-  __shared__ float scratch[16];
+  __shared__ float scratch[32];
   const int t = blockIdx.x;
   const T* src = proj + (size_t)t * proj_stride;
-  const int nqv = nq * hd;
-  float ss = 0.f;
+  const int nqv = nq * hd, nkvv = nkv * hd;
+  // the page is asked for first: its answer comes back while the sums are formed
+  int pos = 0, page = -1;
+  if (has_kv) {
+    pos = positions[t];
+    page = block_table[(size_t)token_entry[t] * bt_stride + pos / page_size];
+  }
+  float ssq = 0.f, ssk = 0.f;
   for (int c = threadIdx.x; c < nqv; c += blockDim.x) {
     const float x = ld_f32(src + q_off + c);
-    ss += x * x;
+    ssq += x * x;
   }
-  float rs = 1.f;
-  if (q_gain) rs = 1.f / sqrtf(block_sum(ss, scratch) / q_count + eps);
+  if (has_kv)
+    for (int c = threadIdx.x; c < nkvv; c += blockDim.x) {
+      const float x = ld_f32(src + k_off + c);
+      ssk += x * x;
+    }
+  block_sum2(ssq, ssk, scratch);
+  const float rsq = q_gain ? 1.f / sqrtf(ssq / q_count + eps) : 1.f;
+  const float rsk = k_gain ? 1.f / sqrtf(ssk / k_count + eps) : 1.f;
   T* qo = q_out + (size_t)t * q_out_stride;
   for (int c = threadIdx.x; c < nqv; c += blockDim.x) {
     const float x = ld_f32(src + q_off + c);
-    st_f32(qo + c, q_gain ? (x * rs) * q_gain[c] : x);
+    st_f32(qo + c, q_gain ? (x * rsq) * q_gain[c] : x);
   }
-  if (!has_kv) return;
-  const int pos = positions[t];
-  const int page = block_table[(size_t)token_entry[t] * bt_stride + pos / page_size];
-  if (page < 0) return;
-  const int nkvv = nkv * hd;
-  ss = 0.f;
-  for (int c = threadIdx.x; c < nkvv; c += blockDim.x) {
-    const float x = ld_f32(src + k_off + c);
-    ss += x * x;
-  }
-  rs = 1.f;
-  if (k_gain) rs = 1.f / sqrtf(block_sum(ss, scratch) / k_count + eps);
+  if (!has_kv || page < 0) return;
   const int slot = pos % page_size;
   for (int c = threadIdx.x; c < nkvv; c += blockDim.x) {
     const int kvh = c / hd, i = c % hd;
     const float x = ld_f32(src + k_off + c);
-    st_f32(k_pool + (((size_t)page * nkv + kvh) * page_size + slot) * hd + i, k_gain ? (x * rs) * k_gain[c] : x);
+    st_f32(k_pool + (((size_t)page * nkv + kvh) * page_size + slot) * hd + i, k_gain ? (x * rsk) * k_gain[c] : x);
     v_pool[(((size_t)page * nkv + kvh) * hd + i) * page_size + slot] = src[v_off + c];
   }
 }

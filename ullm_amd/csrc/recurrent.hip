@@ -140,12 +140,150 @@ ssm_scan_kernel(const float* __restrict__ xbc, const float* __restrict__ proj, i
     for (int e = threadIdx.x; e < N * P; e += SCAN_THREADS) row[e] = S[e];
 }
 
+
+// The same recurrence with the state in registers, for shapes where a thread's share of a column fits there
+// (state rows <= SCAN_NPT * (256 / PC)).  One block per (entry, head, slice of PC columns of the head): thread
+// (r, p) owns rows n = r, r + R, ... of column p.  The entry's tokens are walked in chunks of up to SCAN_CHUNK: a chunk's
+// x, B, C, step sizes and decays are staged in shared memory (the next chunk's loads are issued before the
+// current chunk is worked on and land in the other buffer), every thread moves its rows through the chunk's
+// tokens, leaving one partial sum per token, and after one barrier the block adds each token's R partial sums in
+// the order of r.  A token's result does not depend on where the chunks or the entries are cut: the operations
+// on a state element and their order are the same.
+#define SCAN_NPT 16
+#define SCAN_CHUNK 16
+__global__ void __launch_bounds__(SCAN_THREADS)
+ssm_scan_reg_kernel(const float* __restrict__ xbc, const float* __restrict__ proj, int proj_stride, int dt_off,
+                    const float* __restrict__ dt_bias, const float* __restrict__ a_log, const float* __restrict__ d_skip,
+                    float* __restrict__ state, long long state_stride, long long state_off,
+                    const int* __restrict__ q_start, const int* __restrict__ entry_slot, float* __restrict__ y,
+                    int heads, int groups, int N, int P, int PC, int chunk, int write_state) {
+  extern __shared__ float shared[];
+  const int b = blockIdx.x, h = blockIdx.y, p0 = blockIdx.z * PC, g = h / (heads / groups);
+  const int R = SCAN_THREADS / PC;
+  const int tid = threadIdx.x;
+  const bool active = tid < R * PC;
+  const int p = tid % PC, r = tid / PC;
+  const int per_buf = chunk * (2 * N + PC + 2);          // B | C | x | dt | decay of one chunk
+  float* part = shared + 2 * per_buf;                     // [chunk][R][PC]
+  const int channels = heads * P + 2 * groups * N;
+  const int first = q_start[b], end = q_start[b + 1];
+  float* row = state + (size_t)entry_slot[b] * state_stride + state_off + (size_t)h * N * P + p0;
+  float s[SCAN_NPT];
+#pragma unroll
+  for (int k = 0; k < SCAN_NPT; ++k) {
+    const int n = r + k * R;
+    s[k] = (active && n < N) ? row[(size_t)n * P + p] : 0.f;
+  }
+  const float neg_rate = -expf(a_log[h]);
+  const float bias = dt_bias[h], skip = d_skip[h];
+  const int per_chunk = chunk * (2 * N + PC);             // staged values of a chunk (B, C, x), then chunk step sizes
+  constexpr int STAGE = 20;                                // values a thread stages per chunk, at most
+  // stage(c0, buf): tokens c0 .. c0+chunk-1 of the entry into buffer buf
+  auto fetch = [&](int c0, float (&v)[STAGE]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int u = 0; u < STAGE; ++u) {
+      const int e = tid + u * SCAN_THREADS;
+      float val = 0.f;
+      if (e < per_chunk) {
+        const int t = e / (2 * N + PC), j = e % (2 * N + PC);
+        if (c0 + t < end) {
+          const float* in = xbc + (size_t)(c0 + t) * channels;
+          val = j < N ? in[heads * P + g * N + j]
+                      : (j < 2 * N ? in[heads * P + groups * N + g * N + (j - N)] : in[h * P + p0 + (j - 2 * N)]);
+        }
+      } else if (e < per_chunk + chunk) {
+        const int t = e - per_chunk;
+        val = c0 + t < end ? proj[(size_t)(c0 + t) * proj_stride + dt_off + h] : 0.f;
+      }
+      v[u] = val;
+    }
+  };
+  auto put = [&](const float (&v)[STAGE], float* buf) __attribute__((always_inline)) {
+#pragma unroll
+    for (int u = 0; u < STAGE; ++u) {
+      const int e = tid + u * SCAN_THREADS;
+      if (e < per_chunk) {
+        const int t = e / (2 * N + PC), j = e % (2 * N + PC);
+        buf[t * (2 * N + PC) + j] = v[u];
+      } else if (e < per_chunk + chunk) {
+        const int t = e - per_chunk;
+        const float raw = v[u] + bias;
+        const float dt = raw > 0.f ? raw + log1pf(expf(-raw)) : log1pf(expf(raw));
+        buf[per_chunk + t] = dt;
+        buf[per_chunk + chunk + t] = expf(neg_rate * dt);
+      }
+    }
+  };
+  float v[STAGE];
+  fetch(first, v);
+  put(v, shared);
+  __syncthreads();
+  int turn = 0;
+  for (int c0 = first; c0 < end; c0 += chunk) {
+    float* buf = shared + turn * per_buf;
+    const bool more = c0 + chunk < end;
+    if (more) fetch(c0 + chunk, v);
+    const int n_tok = end - c0 < chunk ? end - c0 : chunk;
+    if (active) {
+      for (int t = 0; t < n_tok; ++t) {
+        const float* bs = buf + t * (2 * N + PC);
+        const float* cs = bs + N;
+        const float dtx = buf[per_chunk + t] * bs[2 * N + p];
+        const float a = buf[per_chunk + chunk + t];
+        float acc = 0.f;
+#pragma unroll
+        for (int k = 0; k < SCAN_NPT; ++k) {
+          const int n = r + k * R;
+          if (n < N) {
+            s[k] = a * s[k] + bs[n] * dtx;
+            acc += s[k] * cs[n];
+          }
+        }
+        part[(t * R + r) * PC + p] = acc;
+      }
+    }
+    __syncthreads();
+    for (int e = tid; e < n_tok * PC; e += SCAN_THREADS) {
+      const int t = e / PC, pp = e % PC;
+      float sum = 0.f;
+      for (int k = 0; k < R; ++k) sum += part[(t * R + k) * PC + pp];
+      y[(size_t)(c0 + t) * heads * P + h * P + p0 + pp] = sum + skip * buf[t * (2 * N + PC) + 2 * N + pp];
+    }
+    if (more) put(v, shared + (1 - turn) * per_buf);
+    __syncthreads();
+    turn = 1 - turn;
+  }
+  if (write_state && active) {
+#pragma unroll
+    for (int k = 0; k < SCAN_NPT; ++k) {
+      const int n = r + k * R;
+      if (n < N) row[(size_t)n * P + p] = s[k];
+    }
+  }
+}
+
 extern "C" int ullm_ssm_scan(const float* xbc, const float* proj, int proj_stride, int dt_off, const float* dt_bias,
                              const float* a_log, const float* d_skip, float* state, long long state_stride,
                              long long state_off, const int* q_start, const int* entry_slot, float* y, int B_,
                              int heads, int groups, int N, int P, int write_state, hipStream_t stream) {
   if (B_ <= 0) return 0;
   if (heads <= 0 || groups <= 0 || heads % groups || N <= 0 || P <= 0 || P > SCAN_THREADS) return ULLM_ERR_SHAPE;
+  // columns of a head per block: 16 where the head cuts into such slices, else the whole head
+  const int PC = P % 16 == 0 ? 16 : P;
+  const int R_reg = SCAN_THREADS / PC;
+  if ((N + R_reg - 1) / R_reg <= SCAN_NPT) {
+    int chunk = SCAN_CHUNK;
+    while (chunk > 1 && ((size_t)chunk * (2 * N + PC) + chunk > 20 * SCAN_THREADS ||
+                         (2 * (size_t)chunk * (2 * N + PC + 2) + (size_t)chunk * R_reg * PC) * sizeof(float) > 64 * 1024))
+      chunk /= 2;
+    const size_t need = (2 * (size_t)chunk * (2 * N + PC + 2) + (size_t)chunk * R_reg * PC) * sizeof(float);
+    if ((size_t)chunk * (2 * N + PC) + chunk <= 20 * SCAN_THREADS && need <= 64 * 1024) {
+      hipLaunchKernelGGL(ssm_scan_reg_kernel, dim3(B_, heads, P / PC), dim3(SCAN_THREADS), need, stream, xbc, proj,
+                         proj_stride, dt_off, dt_bias, a_log, d_skip, state, state_stride, state_off, q_start, entry_slot,
+                         y, heads, groups, N, P, PC, chunk, write_state);
+      ULLM_LAUNCH_CHECK();
+    }
+  }
   int PP = 1;
   while (PP < P) PP *= 2;
   const int R = SCAN_THREADS / PP;
