@@ -225,15 +225,28 @@ def test_scores_scaled_so_that_single_far_keys_stand_out(replayers, models, dtyp
         assert np.median(err) < 3e-2 and err.max() < 0.25, (np.median(err), err.max())
 
 
-def test_kernels_of_the_state_space_mixer_alone():
+# (heads, head size, state, groups, taps, norm parts, tokens of the first step, of the second): sizes that no 16-byte
+# access fits; one row of state a thread; a head that does not cut into whole slices and a state below the rows a
+# block covers, over several staged chunks; the usual sizes; whole heads a block (many heads), with a state that
+# fills the rows and one that does not; a state of many rows a thread
+SSM_SHAPES = [(4, 12, 10, 2, 3, 2, (5, 1, 2), (1, 4, 1)),
+              (4, 16, 8, 2, 4, 2, (5, 1, 2), (1, 4, 1)),
+              (6, 40, 44, 3, 4, 2, (37, 1, 20), (1, 40, 3)),
+              (8, 64, 128, 2, 4, 4, (33, 2, 16), (17, 1, 32)),
+              (344, 64, 24, 8, 2, 8, (18, 1, 2), (1, 21, 1)),
+              (342, 64, 72, 2, 3, 2, (3, 17, 1), (16, 2, 1)),
+              (2, 16, 200, 1, 2, 1, (19, 1, 2), (1, 4, 30))]
+
+
+@pytest.mark.parametrize("heads,P,N,groups,taps,parts,lens1,lens2", SSM_SHAPES)
+def test_kernels_of_the_state_space_mixer_alone(heads, P, N, groups, taps, parts, lens1, lens2):
     """Convolution with carried inputs, the recurrence with carried state, gate and grouped norm: two steps of a
-    batch of three entries against the plain functions run over each entry's whole sequence."""
+    batch of three entries against the plain functions run over each entry's whole sequence.  (In the first shape
+    entry 1 brings fewer tokens than taps-1 and then more.)"""
     from ullm_amd.kernels import ops
     g = torch.Generator().manual_seed(7)
-    heads, P, N, groups, taps, parts = 4, 12, 10, 2, 3, 2
     inner, ch = heads * P, heads * P + 2 * groups * N
     cols = inner + ch + heads
-    lens1, lens2 = (5, 1, 2), (1, 4, 1)                       # entry 1 brings fewer tokens than taps-1 and then more
     conv_w, conv_b = torch.randn(ch, taps, generator=g) * 0.5, torch.randn(ch, generator=g) * 0.2
     dt_bias, a_log, d_skip = (torch.randn(heads, generator=g) * 0.5 for _ in range(3))
     gain = 1 + 0.2 * torch.randn(inner, generator=g)
