@@ -832,14 +832,45 @@ __device__ __forceinline__ ScoreScale split_scale(float scale_log2e) {
 // there was none (m == NEG_BIG counts from zero), it becomes the new one, and the exponents and the output so
 // far are brought to it.  Leaves the weights in `p`, rounded to bfloat16 as they multiply the values, and adds
 // those rounded weights to the sums `l`, two per instruction.
-template <int NQK, int NG, bool masked, bool EXTRA = false, typename KeyOf>
+// With EXTRA the bias row may lie in shared memory (BiasPtr is then a pointer into that address space), and a tile
+// whose keys are all at least `bias_last` behind every column (`bias_far`, the same in the whole wave) adds the
+// row's last value without looking anything up.
+template <int NQK, int NG, bool masked, bool EXTRA = false, typename KeyOf, class BiasPtr = const float*>
 __device__ __forceinline__ void prompt_tile_softmax(f32x4_t (&s)[NG][2], int key0, KeyOf key_of,
                                                     const int (&col_lo)[NG], const int (&col_hi)[NG],
                                                     f32x4_t (&acc)[NG][2 * NQK], float (&m)[NG], f32x4_t (&negm)[NG],
                                                     float (&l)[NG], Pack8 (&p)[NG], const ScoreScale& scale,
-                                                    const float* bias_row = nullptr, int bias_last = 0) {
+                                                    BiasPtr bias_row = nullptr, int bias_last = 0, bool bias_far = false) {
   float lane_max[NG], alpha[NG];
   bool exceeds = false;
+  if constexpr (EXTRA) {
+    if (bias_row && bias_far) {
+      const float far_value = bias_row[bias_last];
+#pragma unroll
+      for (int q = 0; q < NG; ++q)
+#pragma unroll
+        for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) s[q][sb][r] = s[q][sb][r] * scale.frac + far_value;
+    } else if (bias_row) {
+#pragma unroll
+      for (int q = 0; q < NG; ++q)
+#pragma unroll
+        for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {                   // a column's position is the last key it sees
+            const int d = col_hi[q] - (key0 + key_of(sb, r));
+            s[q][sb][r] = s[q][sb][r] * scale.frac + bias_row[d < bias_last ? (d > 0 ? d : 0) : bias_last];
+          }
+    } else {
+#pragma unroll
+      for (int q = 0; q < NG; ++q)
+#pragma unroll
+        for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) s[q][sb][r] *= scale.frac;
+    }
+  }
 #pragma unroll
   for (int q = 0; q < NG; ++q) {
     lane_max[q] = NEG_BIG;
@@ -848,13 +879,7 @@ __device__ __forceinline__ void prompt_tile_softmax(f32x4_t (&s)[NG][2], int key
     for (int sb = 0; sb < 2; ++sb)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        s[q][sb][r] *= scale.frac;                      // the part of scale * log2(e) that is no power of two, in 32-bit
-        if constexpr (EXTRA) {
-          if (bias_row) {                               // a column's position is the last key it sees
-            const int d = col_hi[q] - (key0 + key_of(sb, r));
-            s[q][sb][r] += bias_row[d < bias_last ? (d > 0 ? d : 0) : bias_last];
-          }
-        }
+        if constexpr (!EXTRA) s[q][sb][r] *= scale.frac;  // the part of scale * log2(e) that is no power of two, in 32-bit
         if (masked) {
           const int kk = key0 + key_of(sb, r);
           if (!(kk >= col_lo[q] && kk <= col_hi[q])) s[q][sb][r] = NEG_BIG;
@@ -918,13 +943,13 @@ __device__ __forceinline__ void prompt_tile_softmax(f32x4_t (&s)[NG][2], int key
 // starts from minus the column's reference value over the remaining factor (`negm`, the same in all four
 // elements) instead of zero, so the products times that factor are the exponent itself: exp2 of it is the weight.  A column without a reference
 // value yet (m == NEG_BIG) counts from zero, and the first tile that shows it a key gives it one.
-template <int NQK, int NG, bool masked, bool EXTRA = false>
+template <int NQK, int NG, bool masked, bool EXTRA = false, class BiasPtr = const float*>
 __device__ __forceinline__ void process_tile_lds(const unsigned char* __restrict__ kl, const unsigned char* __restrict__ vl,
                                                  int key0, const Pack8 (&qreg)[NG][NQK],
                                                  const int (&col_lo)[NG], const int (&col_hi)[NG],
                                                  f32x4_t (&acc)[NG][2 * NQK], float (&m)[NG], f32x4_t (&negm)[NG],
                                                  float (&l)[NG], const ScoreScale& scale,
-                                                 const float* bias_row = nullptr, int bias_last = 0) {
+                                                 BiasPtr bias_row = nullptr, int bias_last = 0, bool bias_far = false) {
   using S = PrefillStage<NQK>;
   const int lane = threadIdx.x & 63, g = lane >> 4, c = lane & 15;
   f32x4_t s[NG][2];
@@ -940,7 +965,7 @@ __device__ __forceinline__ void process_tile_lds(const unsigned char* __restrict
     }
   Pack8 p[NG];
   prompt_tile_softmax<NQK, NG, masked, EXTRA>(s, key0, [g](int sb, int r) { return 16 * sb + 4 * g + r; }, col_lo, col_hi,
-                                              acc, m, negm, l, p, scale, bias_row, bias_last);
+                                              acc, m, negm, l, p, scale, bias_row, bias_last, bias_far);
 #pragma unroll
   for (int n = 0; n < 2 * NQK; ++n) {
     Pack8 vf;
@@ -955,7 +980,12 @@ __device__ __forceinline__ void process_tile_lds(const unsigned char* __restrict
 // their own and hand their (reference value, sum, output) to the lower four at the end.  A block then
 // lasts half as long and a compute unit holds one block at a time, so that blocks that finish early
 // (tiles with few keys) make room for the next ones instead of idling beside a long one.
-template <int NQK, int KS, bool EXTRA = false>
+// BIAS_LDS: the block's heads' bias rows are copied to shared memory first ([PREFILL_WAVES][bias_rows] floats of
+// dynamic shared memory), and the scores look them up there.
+typedef const __attribute__((address_space(3))) float* lds_bias_ptr;
+template <bool LDS> struct BiasPointer { typedef const float* type; };
+template <> struct BiasPointer<true> { typedef lds_bias_ptr type; };
+template <int NQK, int KS, bool EXTRA = false, bool BIAS_LDS = false>
 __global__ void __launch_bounds__(64 * PREFILL_WAVES * KS, NQK <= 4 ? 2 / KS : 1)
 attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
                          const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
@@ -988,8 +1018,16 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
   const int head_in_group = (rest % chunks) * PREFILL_WAVES + wave;
   const bool head_ok = head_in_group < G;                 // a wave without a head still helps to load
   const int head = kvh * G + (head_ok ? head_in_group : G - 1);
-  const float* const bias_row = EXTRA && extras.bias ? extras.bias + (size_t)head * extras.bias_rows : nullptr;
+  const float* const bias_global = EXTRA && extras.bias ? extras.bias + (size_t)head * extras.bias_rows : nullptr;
   const int bias_last = extras.bias_rows - 1;
+  extern __shared__ float bias_stage[];
+  if constexpr (BIAS_LDS) {
+    for (int i = lane + 64 * half; i <= bias_last; i += 64 * KS) bias_stage[wave * extras.bias_rows + i] = bias_global[i];
+  }
+  using BiasPtr = typename BiasPointer<BIAS_LDS>::type;
+  BiasPtr bias_row;
+  if constexpr (BIAS_LDS) bias_row = (lds_bias_ptr)bias_stage + wave * extras.bias_rows;
+  else bias_row = bias_global;
   const int first = tiles[2 * tile_idx], count = tiles[2 * tile_idx + 1];
   int clo[NG], chi[NG], tok[NG];
   Pack8 qreg[NG][NQK];
@@ -1058,9 +1096,9 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
   do {                                                                             \
     const unsigned char* kl = tile_lds + (BUF) * TILE_BYTES;                       \
     if ((K0) + 31 > first_pos || (K0) < open_lo)                                   \
-      process_tile_lds<NQK, NG, true, EXTRA>(kl, kl + S::KBYTES, (K0), qreg, clo, chi, acc, m, negm, l, score_scale, bias_row, bias_last);  \
+      process_tile_lds<NQK, NG, true, EXTRA, BiasPtr>(kl, kl + S::KBYTES, (K0), qreg, clo, chi, acc, m, negm, l, score_scale, bias_row, bias_last, EXTRA && (K0) + 31 + bias_last <= first_pos);  \
     else                                                                           \
-      process_tile_lds<NQK, NG, false, EXTRA>(kl, kl + S::KBYTES, (K0), qreg, clo, chi, acc, m, negm, l, score_scale, bias_row, bias_last); \
+      process_tile_lds<NQK, NG, false, EXTRA, BiasPtr>(kl, kl + S::KBYTES, (K0), qreg, clo, chi, acc, m, negm, l, score_scale, bias_row, bias_last, EXTRA && (K0) + 31 + bias_last <= first_pos); \
     STAGE_STORE(NEXT, (K0) + 32, 1 - (BUF));                                       \
     STAGE_LOAD(NEXT, (K0) + 96);                                                   \
     __syncthreads();                                                               \
@@ -1074,9 +1112,9 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
   do {                                                                             \
     const unsigned char* kl = tile_lds + (BUF) * TILE_BYTES;                       \
     if ((K0) + 31 > first_pos || (K0) < open_lo)                                   \
-      process_tile_lds<NQK, NG, true, EXTRA>(kl, kl + S::KBYTES, (K0), qreg, clo, chi, acc, m, negm, l, score_scale, bias_row, bias_last);  \
+      process_tile_lds<NQK, NG, true, EXTRA, BiasPtr>(kl, kl + S::KBYTES, (K0), qreg, clo, chi, acc, m, negm, l, score_scale, bias_row, bias_last, EXTRA && (K0) + 31 + bias_last <= first_pos);  \
     else                                                                           \
-      process_tile_lds<NQK, NG, false, EXTRA>(kl, kl + S::KBYTES, (K0), qreg, clo, chi, acc, m, negm, l, score_scale, bias_row, bias_last); \
+      process_tile_lds<NQK, NG, false, EXTRA, BiasPtr>(kl, kl + S::KBYTES, (K0), qreg, clo, chi, acc, m, negm, l, score_scale, bias_row, bias_last, EXTRA && (K0) + 31 + bias_last <= first_pos); \
   } while (0)
   // Steps go in pairs, so that the two register stages and the two LDS tiles take turns in a way the
   // compiler can see (it then waits for the loads of two steps ago only); an odd last step follows the
@@ -1680,15 +1718,32 @@ extern "C" int ullm_attention_decode_static(
                        block_table, bt_stride, page_size, nq, nkv, hd, scale, window, num_splits, waves, ws, stream);
 }
 
+// `bias_bytes` > 0: the bias rows of a block's heads fit shared memory beside the tiles and are looked up there.
+#define BIAS_STAGE_ROWS 2048
+#define BIAS_STAGE_MAX (PREFILL_WAVES * BIAS_STAGE_ROWS * (int)sizeof(float))
 template <int N, typename... Args>
-static void prefill_launch_extras(int halves, unsigned blocks, hipStream_t stream, Args... args) {
+static void prefill_launch_extras(int halves, size_t bias_bytes, unsigned blocks, hipStream_t stream, Args... args) {
   if constexpr (N <= 4) {
     if (halves == 2) {
-      hipLaunchKernelGGL((attention_prefill_kernel<N, 2, true>), dim3(blocks), dim3(64 * PREFILL_WAVES * 2), 0, stream, args...);
+      if (bias_bytes) {
+        static const hipError_t allowed = hipFuncSetAttribute((const void*)attention_prefill_kernel<N, 2, true, true>,
+                                                              hipFuncAttributeMaxDynamicSharedMemorySize, BIAS_STAGE_MAX);
+        (void)allowed;
+        hipLaunchKernelGGL((attention_prefill_kernel<N, 2, true, true>), dim3(blocks), dim3(64 * PREFILL_WAVES * 2), bias_bytes, stream, args...);
+      }
+      else
+        hipLaunchKernelGGL((attention_prefill_kernel<N, 2, true>), dim3(blocks), dim3(64 * PREFILL_WAVES * 2), 0, stream, args...);
       return;
     }
   }
-  hipLaunchKernelGGL((attention_prefill_kernel<N, 1, true>), dim3(blocks), dim3(64 * PREFILL_WAVES), 0, stream, args...);
+  if (bias_bytes) {
+    static const hipError_t allowed = hipFuncSetAttribute((const void*)attention_prefill_kernel<N, 1, true, true>,
+                                                          hipFuncAttributeMaxDynamicSharedMemorySize, BIAS_STAGE_MAX);
+    (void)allowed;
+    hipLaunchKernelGGL((attention_prefill_kernel<N, 1, true, true>), dim3(blocks), dim3(64 * PREFILL_WAVES), bias_bytes, stream, args...);
+  }
+  else
+    hipLaunchKernelGGL((attention_prefill_kernel<N, 1, true>), dim3(blocks), dim3(64 * PREFILL_WAVES), 0, stream, args...);
 }
 
 template <int N, typename... Args>
@@ -1766,7 +1821,10 @@ static int prefill_any(
 #define CALL(N) prefill_launch<N>(halves, staged, (unsigned)blocks, stream, (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, \
     (const bf16_t*)k_pool, (const bf16_t*)v_pool, tiles, positions, token_entry, block_table, bt_stride, page_size,    \
     nq, nkv, sl, window, n_tiles)
-#define CALL_EXTRA(N) prefill_launch_extras<N>(halves, (unsigned)blocks, stream, (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, \
+  // rows of up to 2048 distances go to shared memory (four heads a block: 32 KiB at most beside the tiles)
+  const size_t bias_bytes = extras && extras->bias && extras->bias_rows <= BIAS_STAGE_ROWS
+                                ? (size_t)PREFILL_WAVES * extras->bias_rows * sizeof(float) : 0;
+#define CALL_EXTRA(N) prefill_launch_extras<N>(halves, bias_bytes, (unsigned)blocks, stream, (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, \
     (const bf16_t*)k_pool, (const bf16_t*)v_pool, tiles, positions, token_entry, block_table, bt_stride, page_size,    \
     nq, nkv, sl, window, n_tiles, *extras)
   if (extras) {
