@@ -208,6 +208,17 @@ ssm_scan_kernel(const float* __restrict__ xbc, const float* __restrict__ proj, i
 #define SCAN_CHUNK 16
 typedef __attribute__((ext_vector_type(4))) float scan_f32x4;
 
+// A barrier for shared memory alone: the block's accesses to shared memory are complete, while loads and stores of
+// global memory stay in flight (the barrier of __syncthreads also waits for those: the next chunk's loads and the
+// results' stores would be waited for twice a chunk).
+__device__ __forceinline__ void shared_memory_barrier() {
+#ifdef __HIP_DEVICE_COMPILE__
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+#endif
+}
+
 template <int PC, int NPT>
 __global__ void __launch_bounds__(SCAN_THREADS)
 ssm_scan_tile_kernel(const float* __restrict__ xbc, const float* __restrict__ proj, int proj_stride, int dt_off,
@@ -283,9 +294,40 @@ ssm_scan_tile_kernel(const float* __restrict__ xbc, const float* __restrict__ pr
       buf[SCAN_CHUNK * ROW + SCAN_CHUNK + tl] = a;
     }
   };
+  struct TokenIn {
+    float b[NPT], c[NPT];
+    float dtx, a;
+  };
+  auto read_token = [&](const float* buf, int t, TokenIn& in) __attribute__((always_inline)) {
+    const float* bs = buf + t * ROW + r * NPT;
+    if constexpr (NPT % 4 == 0) {
+#pragma unroll
+      for (int k = 0; k < NPT; k += 4) {
+        const scan_f32x4 bb = *reinterpret_cast<const scan_f32x4*>(bs + k);
+        const scan_f32x4 cc = *reinterpret_cast<const scan_f32x4*>(bs + NP + k);
+        in.b[k] = bb.x, in.b[k + 1] = bb.y, in.b[k + 2] = bb.z, in.b[k + 3] = bb.w;
+        in.c[k] = cc.x, in.c[k + 1] = cc.y, in.c[k + 2] = cc.z, in.c[k + 3] = cc.w;
+      }
+    } else {
+#pragma unroll
+      for (int k = 0; k < NPT; ++k) in.b[k] = bs[k], in.c[k] = bs[NP + k];
+    }
+    in.dtx = buf[SCAN_CHUNK * ROW + t] * buf[t * ROW + 2 * NP + p];
+    in.a = buf[SCAN_CHUNK * ROW + SCAN_CHUNK + t];
+  };
+  // one token: every row of this thread decays and takes its share of B x; returns the thread's part of y
+  auto move_rows = [&](const TokenIn& in) __attribute__((always_inline)) {
+    float acc = 0.f;
+#pragma unroll
+    for (int k = 0; k < NPT; ++k) {
+      s[k] = in.a * s[k] + in.b[k] * in.dtx;
+      acc += s[k] * in.c[k];
+    }
+    return acc;
+  };
   fetch(first);
   put(first, shared);
-  __syncthreads();
+  shared_memory_barrier();
   int turn = 0;
   for (int c0 = first; c0 < end; c0 += SCAN_CHUNK) {
     const float* buf = shared + turn * PER_BUF;
@@ -293,33 +335,17 @@ ssm_scan_tile_kernel(const float* __restrict__ xbc, const float* __restrict__ pr
     if (more) fetch(c0 + SCAN_CHUNK);
     const int n_tok = end - c0 < SCAN_CHUNK ? end - c0 : SCAN_CHUNK;
     const int t_end = (n_tok + 3) & ~3;
-#pragma unroll 4
-    for (int t = 0; t < t_end; ++t) {
-      const float* bs = buf + t * ROW + r * NPT;
-      const float* cs = bs + NP;
-      const float dtx = buf[SCAN_CHUNK * ROW + t] * buf[t * ROW + 2 * NP + p];
-      const float a = buf[SCAN_CHUNK * ROW + SCAN_CHUNK + t];
-      float acc = 0.f;
-      if constexpr (NPT % 4 == 0) {
-#pragma unroll
-        for (int k = 0; k < NPT; k += 4) {
-          const scan_f32x4 bb = *reinterpret_cast<const scan_f32x4*>(bs + k);
-          const scan_f32x4 cc = *reinterpret_cast<const scan_f32x4*>(cs + k);
-          s[k] = a * s[k] + bb.x * dtx;          acc += s[k] * cc.x;
-          s[k + 1] = a * s[k + 1] + bb.y * dtx;  acc += s[k + 1] * cc.y;
-          s[k + 2] = a * s[k + 2] + bb.z * dtx;  acc += s[k + 2] * cc.z;
-          s[k + 3] = a * s[k + 3] + bb.w * dtx;  acc += s[k + 3] * cc.w;
-        }
-      } else {
-#pragma unroll
-        for (int k = 0; k < NPT; ++k) {
-          s[k] = a * s[k] + bs[k] * dtx;
-          acc += s[k] * cs[k];
-        }
-      }
-      part[(t * R + r) * PC + p] = acc;
+    // a token's B, C, x, step size and decay are read one token ahead of the arithmetic that uses them, into two
+    // sets of registers that take turns: the reads' latency passes while the token before is worked on
+    TokenIn in_a, in_b;
+    read_token(buf, 0, in_a);
+    for (int t = 0; t < t_end; t += 2) {
+      read_token(buf, t + 1, in_b);
+      part[(t * R + r) * PC + p] = move_rows(in_a);
+      read_token(buf, t + 2 < SCAN_CHUNK ? t + 2 : SCAN_CHUNK - 1, in_a);
+      part[((t + 1) * R + r) * PC + p] = move_rows(in_b);
     }
-    __syncthreads();
+    shared_memory_barrier();
     for (int e = tid; e < n_tok * PC; e += SCAN_THREADS) {
       const int t = e / PC, pp = e % PC;
       if (p0 + pp < P) {
@@ -330,7 +356,7 @@ ssm_scan_tile_kernel(const float* __restrict__ xbc, const float* __restrict__ pr
       }
     }
     if (more) put(c0 + SCAN_CHUNK, shared + (1 - turn) * PER_BUF);
-    __syncthreads();
+    shared_memory_barrier();
     turn = 1 - turn;
   }
   if (write_state && column) {
