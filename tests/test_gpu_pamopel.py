@@ -54,8 +54,14 @@ CFG_R = config(32, 64, [mamba(2, 8, 24, 1, 1, 2), attn(2, 2, 8, 16, 30, 0.5, ff=
 CFG_S = config(32, 50, [attn(2, 1, 16, 16, 100, 6.0, ff=40), attn(2, 1, 16, 16, 100, 6.0, kv_from=0)])
 # B: a distance table that decides every weight (queries scaled away)
 CFG_B = config(32, 50, [attn(3, 1, 16, 16, 37, 0.01)])
+# T: head sizes the matrix-core kernels take, keys and values of different size (32 | 64 and 64 | 32), a state-space
+# layer first and last with sizes that cut into 16-byte pieces (the vector convolution, the register scan), a
+# feed-forward behind one of them, three query heads a key head
+CFG_T = config(64, 113, [mamba(4, 16, 16, 2, 4, 2, ff=96), attn(6, 2, 32, 64, 64, 0.2, ff=96),
+                         attn(6, 2, 32, 64, 64, 0.2, kv_from=1), attn(4, 4, 64, 32, 20, 0.15), mamba(4, 16, 64, 1, 3, 1)],
+               bigram=(251, 5, 11), mult=0.7)
 MODELS = {"P": (CFG_P, 1, 32, 1.0), "Q": (CFG_Q, 2, 6, 1.0), "R": (CFG_R, 3, 32, 1.0), "S": (CFG_S, 4, 32, 0.1),
-          "B": (CFG_B, 5, 13, 4.0)}
+          "B": (CFG_B, 5, 13, 4.0), "T": (CFG_T, 6, 24, 1.0)}
 
 
 @pytest.fixture(scope="module")
@@ -84,7 +90,7 @@ def oracle(models, name, toks):
 
 
 def close(got, want, dtype, name=""):
-    if dtype == "bfloat16" and name in ("P", "Q", "R"):
+    if dtype == "bfloat16" and name in ("P", "Q", "R", "T"):
         # A state-space layer norms its gated output in parts, and the block norms the branch again: at a token where
         # a part happens to be ten times smaller than usual, the rounding of the layer's input comes out ten times
         # larger (seen: one row of 75 at 6e-2 of the largest logit where the 64-bit implementation with weights
@@ -130,7 +136,7 @@ def run(rep, rid, toks, cuts, end=True):
     return np.concatenate(got)
 
 
-CASES = [(n, d) for n in ("P", "Q", "R") for d in ("float32", "bfloat16")]
+CASES = [(n, d) for n in ("P", "Q", "R", "T") for d in ("float32", "bfloat16")]
 
 
 @pytest.mark.parametrize("name,dtype", CASES)
@@ -341,7 +347,7 @@ def test_norm_behind_a_branch_the_add_and_the_next_norm_in_one_pass(kind, post_k
         assert torch.equal(some, got[[3, 0]]) and torch.equal(r2.cpu(), res)
 
 
-@pytest.mark.parametrize("name", ["P", "Q"])
+@pytest.mark.parametrize("name", ["P", "Q", "T"])
 def test_greedy_generation_through_the_entry_point(models, name):
     from ullm_amd import LLM, EngineConfig, SamplingParams
     d, cfg, w = models[name]
