@@ -466,7 +466,7 @@ def test_bfloat16_prefix_cache_along_each_requests_own_path(tmp_path):
         return launch(prepared)
     eng.runner.launch = counting
     prompts = [shared + [9], shared[:33] + [7, 7], other, shared + [1, 2, 3, 4]]
-    for i, p in enumerate(prompts):                      # under fresh ids: the checker names requests r0, r1, ...
+    for i, p in enumerate(prompts):                      # under fresh ids r0, r1, ...
         eng.add_request(f"r{i}", p, sp)
     got = {}
     seen = {}
