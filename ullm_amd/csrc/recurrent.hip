@@ -285,9 +285,13 @@ ssm_scan_tile_kernel(const float* __restrict__ xbc, const float* __restrict__ pr
     if (ln == 15) {
       float dt = 0.f, a = 1.f;
       if (c0 + tl < end) {
-        // softplus without a clamp: log(1 + e^raw), written so that neither side overflows
+        // softplus without a clamp: max(raw, 0) + log(1 + e^-|raw|), one exponential and one logarithm;
+        // log(u) * e / (u - 1) with u = 1 + e rounded is log(1 + e) to a few units in the last place for any e
+        // (every wave has such lanes, so whatever stands here is issued by all of them once a chunk)
         const float raw = vdt + bias;
-        dt = raw > 0.f ? raw + log1pf(expf(-raw)) : log1pf(expf(raw));
+        const float e = expf(-fabsf(raw)), u = 1.f + e;
+        const float l = u == 1.f ? e : logf(u) * (e / (u - 1.f));
+        dt = fmaxf(raw, 0.f) + l;
         a = expf(neg_rate * dt);
       }
       buf[SCAN_CHUNK * ROW + tl] = dt;
