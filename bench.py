@@ -146,7 +146,7 @@ def design_configs(shape):
         else:
             layers.append(dict(type="attention", mlp=mlp, mixer=dict(att, kv_from=i - 1) if kind == 1 else dict(att)))
     pamopel = dict(architecture="Pamopel", vocab=DESIGN_VOCAB, width=W, layers=layers, norm=dict(eps=1e-5), residual_mult=0.5,
-                   logit_scale=1.0, embedding=dict(scale=1.0, bigram=dict(buckets=65521, mul_prev=31, mul_cur=17)))
+                   logit_scale=1.0, embedding=dict(scale=1.0, bigram=dict(buckets=65521, mul_prev=8191, mul_cur=127)))
     qwen = dict(architectures=["Qwen3ForCausalLM"], hidden_size=W, num_hidden_layers=L, num_attention_heads=H,
                 num_key_value_heads=G, head_dim=D, intermediate_size=F, vocab_size=DESIGN_VOCAB, rope_theta=1e6,
                 rms_norm_eps=1e-6, max_position_embeddings=40960, tie_word_embeddings=False, attention_bias=False,

@@ -376,8 +376,9 @@ def test_the_trace_program_runs_the_design(models, trace_run):
     close(np.concatenate((a, b)), want[[0, 20, 39]], "float32")
 
 
-@pytest.mark.parametrize("hd,nq,nkv", [(64, 8, 1), (128, 6, 2), (32, 20, 1), (96, 4, 4), (256, 2, 1)])
-def test_matrix_core_attention_with_distance_bias_and_head_gates(hd, nq, nkv):
+@pytest.mark.parametrize("rows", [70, 2100])        # 2100: more distances than the prompt kernel keeps in shared memory
+@pytest.mark.parametrize("hd,nq,nkv", [(64, 10, 2), (128, 6, 2), (32, 20, 1), (96, 4, 4), (256, 2, 1)])
+def test_matrix_core_attention_with_distance_bias_and_head_gates(hd, nq, nkv, rows):
     """The bfloat16 kernels (single tokens cut over splits and their reduce; prompt tiles) against 64-bit softmax
     attention on the same rounded operands: a bias by distance whose entries are units apart, clamped at the
     table's last entry, and a gate per head; contexts that end at and beside tile and page borders, one past 1 100
@@ -390,7 +391,6 @@ def test_matrix_core_attention_with_distance_bias_and_head_gates(hd, nq, nkv):
     from ullm_amd.parts.attention import plan_attention_step
     g = torch.Generator().manual_seed(hd + nq)
     starts, lens = [1130, 31, 64, 200, 0], [1, 1, 1, 45, 33]            # tokens before the step, new tokens
-    rows = 70
     bias = (torch.randn(nq, rows, generator=g) * 2).float()
     seqs_k = [torch.randn(s + n, nkv, hd, generator=g).bfloat16().float() for s, n in zip(starts, lens)]
     seqs_v = [torch.randn(s + n, nkv, hd, generator=g).bfloat16().float() for s, n in zip(starts, lens)]
