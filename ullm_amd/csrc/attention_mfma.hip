@@ -1297,12 +1297,13 @@ __device__ __forceinline__ void dma_tile_load(unsigned char* tile, int key0, int
 
 // Scores, softmax update and value product of one wave for the tile in shared memory; as process_tile_lds,
 // with the keys' order and the tile's layout as described above.
-template <int NQK, int NG, bool masked>
+template <int NQK, int NG, bool masked, bool EXTRA = false, class BiasPtr = const float*>
 __device__ __forceinline__ void dma_tile_products(const unsigned char* __restrict__ tile, int key0, const Pack8 (&qreg)[NG][NQK],
                                                   const int (&col_lo)[NG], const int (&col_hi)[NG],
                                                   f32x4_t (&acc)[NG][2 * NQK], float (&m)[NG], f32x4_t (&negm)[NG],
                                                   float (&l)[NG], const int (&k_at)[2][NQK], int v_at, int max_hi,
-                                                  bool ok0, bool ok1, const ScoreScale& scale) {
+                                                  bool ok0, bool ok1, const ScoreScale& scale,
+                                                  BiasPtr bias_row = nullptr, int bias_last = 0, bool bias_far = false) {
   using T = DmaTile<NQK>;
   const int lane = threadIdx.x & 63, g = lane >> 4;
   f32x4_t s[NG][2];
@@ -1318,8 +1319,8 @@ __device__ __forceinline__ void dma_tile_products(const unsigned char* __restric
     }
   // s[q][sb][r] is the exponent of key key0 + 8 g + 4 sb + r for this lane's column
   Pack8 p[NG];
-  prompt_tile_softmax<NQK, NG, masked>(s, key0, [g](int sb, int r) { return 8 * g + 4 * sb + r; }, col_lo, col_hi,
-                                       acc, m, negm, l, p, scale);
+  prompt_tile_softmax<NQK, NG, masked, EXTRA>(s, key0, [g](int sb, int r) { return 8 * g + 4 * sb + r; }, col_lo, col_hi,
+                                              acc, m, negm, l, p, scale, bias_row, bias_last, bias_far);
   // masked tiles only: which of this lane's eight keys (8 g ..) hold written values.  The others (past the end
   // of the data, or in a sub-block without a page, which reads page 0) may hold anything and must count as 0.
   uint32_t live[4] = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu};
@@ -1344,14 +1345,16 @@ __device__ __forceinline__ void dma_tile_products(const unsigned char* __restric
   }
 }
 
-template <int NQK, int KS>
+// EXTRA: a bias by distance (never null here; the block's four heads' rows are copied to dynamic shared memory
+// first, [PREFILL_WAVES][bias_rows] floats) and the gate per head, as in attention_prefill_kernel.
+template <int NQK, int KS, bool EXTRA = false>
 __global__ void __launch_bounds__(64 * PREFILL_WAVES * KS, 2 / KS)
 attention_prefill_dma_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
                              const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
                              const int* __restrict__ tiles, const int* __restrict__ positions,
                              const int* __restrict__ token_entry, const int* __restrict__ block_table,
                              int bt_stride, int page_size, int nq, int nkv, float scale_log2e, int window,
-                             int n_tiles) {
+                             int n_tiles, ScoreExtras extras) {
   using T = DmaTile<NQK>;
   constexpr int HD = 32 * NQK;
   constexpr int NG = PREFILL_GROUPS;
@@ -1380,6 +1383,15 @@ attention_prefill_dma_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t*
   const int head_in_group = (rest % chunks) * PREFILL_WAVES + wave;
   const bool head_ok = head_in_group < G;                 // a wave without a head still helps to load
   const int head = kvh * G + (head_ok ? head_in_group : G - 1);
+  extern __shared__ float dma_bias_stage[];
+  const int bias_last = extras.bias_rows - 1;
+  using BiasPtr = typename BiasPointer<EXTRA>::type;
+  BiasPtr bias_row = nullptr;
+  if constexpr (EXTRA) {
+    const float* const bias_global = extras.bias + (size_t)head * extras.bias_rows;
+    for (int i = lane + 64 * half; i <= bias_last; i += 64 * KS) dma_bias_stage[wave * extras.bias_rows + i] = bias_global[i];
+    bias_row = (lds_bias_ptr)dma_bias_stage + wave * extras.bias_rows;
+  }
   const int first = tiles[2 * tile_idx], count = tiles[2 * tile_idx + 1];
   int clo[NG], chi[NG], tok[NG];
   Pack8 qreg[NG][NQK];
@@ -1474,9 +1486,11 @@ attention_prefill_dma_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t*
       if (i + 3 < steps) TILE_LOAD(i + 3, t0);
       if (K0 + 31 > first_pos || K0 < open_lo) {
         const bool ok0 = pages[2 * (i - t0)] >= 0, ok1 = pages[2 * (i - t0) + 1] >= 0;
-        dma_tile_products<NQK, NG, true>(tile, K0, qreg, clo, chi, acc, m, negm, l, k_at, v_at, last_pos, ok0, ok1, score_scale);
+        dma_tile_products<NQK, NG, true, EXTRA, BiasPtr>(tile, K0, qreg, clo, chi, acc, m, negm, l, k_at, v_at, last_pos, ok0, ok1,
+                                                         score_scale, bias_row, bias_last, EXTRA && K0 + 31 + bias_last <= first_pos);
       } else {
-        dma_tile_products<NQK, NG, false>(tile, K0, qreg, clo, chi, acc, m, negm, l, k_at, v_at, last_pos, true, true, score_scale);
+        dma_tile_products<NQK, NG, false, EXTRA, BiasPtr>(tile, K0, qreg, clo, chi, acc, m, negm, l, k_at, v_at, last_pos, true, true,
+                                                          score_scale, bias_row, bias_last, EXTRA && K0 + 31 + bias_last <= first_pos);
       }
     }
   }
@@ -1521,7 +1535,8 @@ attention_prefill_dma_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t*
     lt += __shfl_xor(lt, 16, 64);
     lt += __shfl_xor(lt, 32, 64);
     if (chi[qg] < 0) continue;
-    const float inv = lt > 0.f ? 1.f / lt : 0.f;
+    float inv = lt > 0.f ? 1.f / lt : 0.f;
+    if constexpr (EXTRA) inv *= gate_of(extras, tok[qg], head);
     bf16_t* op = out + (size_t)tok[qg] * out_stride + (size_t)head * HD;
 #pragma unroll
     for (int n = 0; n < 2 * NQK; ++n)
@@ -1721,8 +1736,25 @@ extern "C" int ullm_attention_decode_static(
 // `bias_bytes` > 0: the bias rows of a block's heads fit shared memory beside the tiles and are looked up there.
 #define BIAS_STAGE_ROWS 2048
 #define BIAS_STAGE_MAX (PREFILL_WAVES * BIAS_STAGE_ROWS * (int)sizeof(float))
+#define DMA_BIAS_ROWS 1792                // what fits beside four tiles a half and the page ids, for both halves
 template <int N, typename... Args>
 static void prefill_launch_extras(int halves, size_t bias_bytes, unsigned blocks, hipStream_t stream, Args... args) {
+  if constexpr (N == 4) {                 // tiles straight to shared memory, as without extras
+    if (bias_bytes && bias_bytes <= (size_t)PREFILL_WAVES * DMA_BIAS_ROWS * sizeof(float)) {
+      if (halves == 2) {
+        static const hipError_t allowed = hipFuncSetAttribute((const void*)attention_prefill_dma_kernel<N, 2, true>,
+            hipFuncAttributeMaxDynamicSharedMemorySize, PREFILL_WAVES * DMA_BIAS_ROWS * (int)sizeof(float));
+        (void)allowed;
+        hipLaunchKernelGGL((attention_prefill_dma_kernel<N, 2, true>), dim3(blocks), dim3(64 * PREFILL_WAVES * 2), bias_bytes, stream, args...);
+      } else {
+        static const hipError_t allowed = hipFuncSetAttribute((const void*)attention_prefill_dma_kernel<N, 1, true>,
+            hipFuncAttributeMaxDynamicSharedMemorySize, PREFILL_WAVES * DMA_BIAS_ROWS * (int)sizeof(float));
+        (void)allowed;
+        hipLaunchKernelGGL((attention_prefill_dma_kernel<N, 1, true>), dim3(blocks), dim3(64 * PREFILL_WAVES), bias_bytes, stream, args...);
+      }
+      return;
+    }
+  }
   if constexpr (N <= 4) {
     if (halves == 2) {
       if (bias_bytes) {
@@ -1752,9 +1784,9 @@ static void prefill_launch(int halves, bool staged, unsigned blocks, hipStream_t
   if constexpr (N == 4) {
     if (!staged) {                                        // tiles straight to shared memory
       if (halves == 2)
-        hipLaunchKernelGGL((attention_prefill_dma_kernel<N, 2>), dim3(blocks), dim3(64 * PREFILL_WAVES * 2), 0, stream, args...);
+        hipLaunchKernelGGL((attention_prefill_dma_kernel<N, 2>), dim3(blocks), dim3(64 * PREFILL_WAVES * 2), 0, stream, args..., none);
       else
-        hipLaunchKernelGGL((attention_prefill_dma_kernel<N, 1>), dim3(blocks), dim3(64 * PREFILL_WAVES), 0, stream, args...);
+        hipLaunchKernelGGL((attention_prefill_dma_kernel<N, 1>), dim3(blocks), dim3(64 * PREFILL_WAVES), 0, stream, args..., none);
       return;
     }
   }
