@@ -295,3 +295,119 @@ class PamopelConfig:
     @property
     def num_hidden_layers(self) -> int:
         return len(self.layers)
+
+
+@dataclass(frozen=True)
+class ZiferaxAttention:
+    """Sizes and constants of one Ziferax attention mixer."""
+    heads: int
+    kv_heads: int
+    dim: int                        # per-head query / key size; the values are the keys, so also the value size
+    scale: float
+    window: int                     # keys a query sees, itself included; 0: all
+    rot_dims: int                   # leading dims of each head that are rotated; 0: none
+    rot_base: float
+
+
+@dataclass(frozen=True)
+class ZiferaxExperts:
+    """Sizes and constants of one Ziferax routed feed-forward."""
+    experts: int                    # experts with tensors
+    identity: int                   # router outputs beyond them whose expert returns its input
+    top: int
+    ff: int
+    limit: float
+    shared_ff: int                  # 0: no shared expert
+    shared_limit: float
+
+
+@dataclass(frozen=True)
+class ZiferaxLayer:
+    type: str
+    mixer: ZiferaxAttention
+    mlp: Optional[ZiferaxExperts]
+    weights_of: Optional[int]       # the layer whose tensors this one uses (with a cache of its own), or None
+
+
+@dataclass(frozen=True)
+class ZiferaxConfig:
+    """Keys of a Ziferax config.json: a stack of parallel blocks (one RMS norm, attention and a routed
+    feed-forward that both read it, a multiplier on their sum), listed layer by layer.  Attention has biases on
+    q, k and the output, values that are the keys before rotation, rotation of adjacent pairs over the heads' first
+    ``rot.dims`` dims, a sliding window and a sink per head.  A layer with ``weights_of`` uses another layer's
+    tensors.  The head is the embedding table."""
+    architecture: str
+    vocab_size: int
+    hidden_size: int
+    layers: tuple                   # of ZiferaxLayer
+    norm_eps: float
+    residual_mult: float
+
+    @classmethod
+    def from_dict(cls, d: Mapping[str, Any]) -> "ZiferaxConfig":
+        norm = d.get("norm") or {}
+        raw_layers = d.get("layers")
+        if not isinstance(raw_layers, (list, tuple)) or not raw_layers:
+            raise ConfigError("config.json: key 'layers' must be a non-empty list")
+        layers = []
+        for i, L in enumerate(raw_layers):
+            try:
+                if not isinstance(L, Mapping):
+                    raise ConfigError("a layer must be an object")
+                kind = _take(L, "type", str)
+                if kind != "attention":
+                    raise ConfigError(f"type {kind!r}; known: ['attention']")
+                m = L.get("mixer")
+                if not isinstance(m, Mapping):
+                    raise ConfigError("no 'mixer' object")
+                mask, rot = m.get("mask") or {}, m.get("rot") or {}
+                dim = _take(m, "dim", int)
+                att = ZiferaxAttention(
+                    heads=_take(m, "heads", int), kv_heads=_take(m, "kv_heads", int), dim=dim,
+                    scale=_take(m, "scale", float), window=_take(mask, "size", int, 0),
+                    rot_dims=_take(rot, "dims", int, 0), rot_base=_take(rot, "base", float, 10000.0))
+                if _take(m, "vdim", int, dim) != dim:
+                    raise ConfigError(f"'vdim' = {m['vdim']} differs from 'dim' = {dim}: the values are the keys")
+                if att.heads < 1 or att.kv_heads < 1 or att.heads % att.kv_heads or dim < 1:
+                    raise ConfigError(f"{att.heads} heads over {att.kv_heads} kv heads of size {dim}")
+                if att.rot_dims < 0 or att.rot_dims % 2 or att.rot_dims > dim or att.window < 0:
+                    raise ConfigError(f"rot.dims = {att.rot_dims} must be even and at most dim = {dim}; mask.size >= 0")
+                mlp = L.get("mlp")
+                if mlp is not None:
+                    if not isinstance(mlp, Mapping) or _take(mlp, "kind", str) != "moe":
+                        raise ConfigError("'mlp' must be null or an object of kind 'moe'")
+                    router, expert = mlp.get("router") or {}, mlp.get("expert") or {}
+                    shared = mlp.get("shared") or {}
+                    mlp = ZiferaxExperts(
+                        experts=_take(router, "experts", int), identity=_take(router, "identity", int, 0),
+                        top=_take(router, "top", int), ff=_take(expert, "ff", int), limit=_take(expert, "limit", float),
+                        shared_ff=_take(shared, "ff", int, 0),
+                        shared_limit=_take(shared, "limit", float, _take(expert, "limit", float)))
+                    if mlp.experts < 0 or mlp.identity < 0 or not 1 <= mlp.top <= mlp.experts + mlp.identity:
+                        raise ConfigError(f"top = {mlp.top} of {mlp.experts} experts and {mlp.identity} identity experts")
+                    if (mlp.experts and mlp.ff < 1) or mlp.shared_ff < 0 or not mlp.limit > 0 or not mlp.shared_limit > 0:
+                        raise ConfigError("expert sizes and limits must be positive")
+                src = L.get("weights_of")
+                if src is not None:
+                    src = _take(L, "weights_of", int)
+                    if not 0 <= src < len(raw_layers) or src == i or raw_layers[src].get("weights_of") is not None:
+                        raise ConfigError(f"'weights_of': {src} must name another layer with tensors of its own")
+            except ConfigError as e:
+                raise ConfigError(f"{e} (layer {i})") from None
+            layers.append(ZiferaxLayer(kind, att, mlp, src))
+        for i, L in enumerate(layers):
+            if L.weights_of is not None:
+                o = layers[L.weights_of]
+                if (o.mixer, o.mlp) != (L.mixer, L.mlp):
+                    raise ConfigError(f"config.json: layer {i} uses the tensors of layer {L.weights_of} but their "
+                                      f"entries differ")
+        cfg = cls(architecture=_take(d, "architecture", str, "Ziferax"), vocab_size=_take(d, "vocab", int),
+                  hidden_size=_take(d, "width", int), layers=tuple(layers), norm_eps=_take(norm, "eps", float),
+                  residual_mult=_take(d, "residual_mult", float, 1.0))
+        if cfg.vocab_size < 1 or cfg.hidden_size < 1 or cfg.norm_eps < 0:
+            raise ConfigError("config.json: 'vocab' and 'width' must be positive and 'norm.eps' not negative")
+        return cfg
+
+    @property
+    def num_hidden_layers(self) -> int:
+        return len(self.layers)

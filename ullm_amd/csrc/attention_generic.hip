@@ -4,7 +4,8 @@
 // that depends only on the token's own position, so the result for a token is the same however
 // the batch was cut.  Scores, running maximum, sum and output are 32-bit.  Optionally a bias by
 // distance is added to every score: bias[head, min(query position - key position, bias_rows - 1)]
-// (float32 [nq, bias_rows]); the scale does not multiply it.
+// (float32 [nq, bias_rows]); the scale does not multiply it.  Optionally a sink per head (float32 [nq]): one more
+// term exp(sink[head]) in the softmax's denominator that has no key and no value and is not scaled.
 // Pools: keys [page, kv_head, row, head_dim]; values [page, kv_head, head_dim, row].
 //
 // Semantics as the reference asks of its attention library (ullm/layers/attention.py:76-104,
@@ -22,7 +23,8 @@ paged_attention_generic_kernel(const T* __restrict__ q, int q_stride, T* __restr
                                const int* __restrict__ positions, const int* __restrict__ token_entry,
                                const int* __restrict__ block_table, int bt_stride, int page_size,
                                int nq, int nkv, int hd, float scale, int window,
-                               const float* __restrict__ bias, int bias_rows) {
+                               const float* __restrict__ bias, int bias_rows,
+                               const float* __restrict__ sink) {
   __shared__ float q_s[ATT_MAX_HD];
   __shared__ float p_s[ATT_THREADS];
   __shared__ long long row_s[ATT_THREADS];
@@ -87,7 +89,15 @@ paged_attention_generic_kernel(const T* __restrict__ q, int q_stride, T* __restr
     if (m_new > -INFINITY) m = m_new;
   }
   T* op = out + (size_t)t * out_stride + (size_t)h * hd;
-  const float inv = l > 0.f ? 1.f / l : 0.f;
+  float keep = 1.f;
+  if (sink) {
+    // the sink joins the denominator alone: sum and outputs move to the larger of the two reference values
+    const float sv = sink[h];
+    const float m_all = fmaxf(m, sv);
+    keep = (m == -INFINITY) ? 0.f : expf(m - m_all);
+    l = l * keep + expf(sv - m_all);
+  }
+  const float inv = l > 0.f ? keep / l : 0.f;
 #pragma unroll
   for (int r = 0; r < DPT; ++r) {
     const int d = tid + r * ATT_THREADS;
@@ -98,8 +108,8 @@ paged_attention_generic_kernel(const T* __restrict__ q, int q_stride, T* __restr
 extern "C" int ullm_paged_attention_generic(
     const void* q, int q_stride, void* out, int out_stride, const void* k_pool, const void* v_pool,
     const int* positions, const int* token_entry, const int* block_table, int bt_stride, int page_size,
-    int T_, int nq, int nkv, int hd, float scale, int window, const float* bias, int bias_rows, int dtype,
-    hipStream_t stream) {
+    int T_, int nq, int nkv, int hd, float scale, int window, const float* bias, int bias_rows,
+    const float* sink, int dtype, hipStream_t stream) {
   if (T_ <= 0) return 0;
   if (bias && bias_rows <= 0) return ULLM_ERR_SHAPE;
   if (hd <= 0 || hd > ATT_MAX_HD || nq <= 0 || nkv <= 0 || nq % nkv != 0 || page_size <= 0 || window < 0)
@@ -107,7 +117,7 @@ extern "C" int ullm_paged_attention_generic(
   dim3 grid(T_, nq), block(ATT_THREADS);
 #define GO(TT) hipLaunchKernelGGL(paged_attention_generic_kernel<TT>, grid, block, 0, stream, \
     (const TT*)q, q_stride, (TT*)out, out_stride, (const TT*)k_pool, (const TT*)v_pool, positions, \
-    token_entry, block_table, bt_stride, page_size, nq, nkv, hd, scale, window, bias, bias_rows)
+    token_entry, block_table, bt_stride, page_size, nq, nkv, hd, scale, window, bias, bias_rows, sink)
   if (dtype == ULLM_F32) GO(float);
   else if (dtype == ULLM_BF16) GO(bf16_t);
   else return ULLM_ERR_DTYPE;

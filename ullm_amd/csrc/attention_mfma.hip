@@ -106,13 +106,20 @@ __device__ __forceinline__ void load_tile(KVTile<NQK>& t, int key0, const PageWi
 // What the variants with EXTRA add to a score and to a head's output: a bias by distance, bias[head][min(query
 // position - key position, last)] in units of log2 (the caller multiplies its table by log2(e) once: the scores
 // are exponents of two), added to the scaled score in 32-bit; and a gate per head, sigmoid(gate[token][head]),
-// that multiplies the head's normalised output on its way out.  Either pointer may be null.
+// that multiplies the head's normalised output on its way out; and a sink per head, one more term 2^sink[head]
+// in the softmax's denominator (units of log2 again: the caller multiplies by log2(e)) that has no key and no
+// value.  Any pointer may be null.
 struct ScoreExtras {
   const float* bias;          // [nq][bias_rows]
   int bias_rows;
   const bf16_t* gate;         // [tokens][gate_stride], one value per head
   int gate_stride;
+  const float* sink;          // [nq]
 };
+// What the sink adds to a sum of weights taken relative to the exponent `reference`.
+__device__ __forceinline__ float sink_of(const ScoreExtras& x, int head, float reference) {
+  return x.sink ? fast_exp2(x.sink[head] - reference) : 0.f;
+}
 __device__ __forceinline__ float gate_of(const ScoreExtras& x, int token, int head) {
   if (!x.gate) return 1.f;
   return 1.f / (1.f + __expf(-bf16_bits_to_f32(x.gate[(size_t)token * x.gate_stride + head])));
@@ -595,6 +602,7 @@ attention_decode_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __re
   l += __shfl_xor(l, 32, 64);
   if (!col_ok) return;
   if (num_splits == 1) {
+    if constexpr (EXTRA) l += sink_of(extras, head, m);
     float inv = l > 0.f ? 1.f / l : 0.f;
     if constexpr (EXTRA) inv *= gate_of(extras, t, head);
     bf16_t* op = out + (size_t)t * out_stride + (size_t)head * HD;
@@ -665,6 +673,7 @@ attention_reduce_kernel(const float* __restrict__ part, bf16_t* __restrict__ out
       }
     }
   }
+  L += sink_of(extras, head, M);
   const float inv = (L > 0.f ? 1.f / L : 0.f) * gate_of(extras, t, head);
   bf16_t* op = out + (size_t)t * out_stride + (size_t)head * hd;
 #pragma unroll
@@ -1176,6 +1185,7 @@ attention_prefill_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t* __r
     lt += __shfl_xor(lt, 16, 64);
     lt += __shfl_xor(lt, 32, 64);
     if (chi[qg] < 0) continue;
+    if constexpr (EXTRA) lt += sink_of(extras, head, m[qg]);
     float inv = lt > 0.f ? 1.f / lt : 0.f;
     if constexpr (EXTRA) inv *= gate_of(extras, tok[qg], head);
     bf16_t* op = out + (size_t)tok[qg] * out_stride + (size_t)head * HD;
@@ -1535,6 +1545,7 @@ attention_prefill_dma_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t*
     lt += __shfl_xor(lt, 16, 64);
     lt += __shfl_xor(lt, 32, 64);
     if (chi[qg] < 0) continue;
+    if constexpr (EXTRA) lt += sink_of(extras, head, m[qg]);
     float inv = lt > 0.f ? 1.f / lt : 0.f;
     if constexpr (EXTRA) inv *= gate_of(extras, tok[qg], head);
     bf16_t* op = out + (size_t)tok[qg] * out_stride + (size_t)head * HD;
@@ -1627,14 +1638,15 @@ static int decode_launch(
 }
 
 // ullm_attention_decode with a bias by distance on the scores (float32 [nq][bias_rows], already multiplied by
-// log2(e); null for none) and a gate per head on the outputs (bfloat16 [tokens][gate_stride]; null for none).
+// log2(e); null for none), a gate per head on the outputs (bfloat16 [tokens][gate_stride]; null for none) and a
+// sink per head in the softmax's denominator (float32 [nq], already multiplied by log2(e); null for none).
 extern "C" int ullm_attention_decode_extras(
     const void* q, int q_stride, void* out, int out_stride, const void* k_pool, const void* v_pool,
     const int* token_list, int n_items, const int* positions, const int* token_entry,
     const int* block_table, int bt_stride, int page_size, int nq, int nkv, int hd, float scale, int window,
     int num_splits, int waves, float* workspace, const float* bias, int bias_rows, const void* gate, int gate_stride,
-    hipStream_t stream) {
-  const ScoreExtras x{bias, bias_rows, (const bf16_t*)gate, gate_stride};
+    const float* sink, hipStream_t stream) {
+  const ScoreExtras x{bias, bias_rows, (const bf16_t*)gate, gate_stride, sink};
   return decode_launch(q, q_stride, out, out_stride, k_pool, v_pool, token_list, n_items, positions, token_entry,
                        block_table, bt_stride, page_size, nq, nkv, hd, scale, window, num_splits, waves, workspace,
                        stream, nullptr, &x);
@@ -1885,8 +1897,8 @@ extern "C" int ullm_attention_prefill_extras(
     const int* tiles, int n_tiles, const int* positions, const int* token_entry, const int* block_table,
     int bt_stride, int page_size, int nq, int nkv, int hd, float scale, int window, int halves,
     long long keys_total, int keys_max, const float* bias, int bias_rows, const void* gate, int gate_stride,
-    hipStream_t stream) {
-  const ScoreExtras x{bias, bias_rows, (const bf16_t*)gate, gate_stride};
+    const float* sink, hipStream_t stream) {
+  const ScoreExtras x{bias, bias_rows, (const bf16_t*)gate, gate_stride, sink};
   return prefill_any(q, q_stride, out, out_stride, k_pool, v_pool, tiles, n_tiles, positions, token_entry, block_table,
                      bt_stride, page_size, nq, nkv, hd, scale, window, halves % 10, keys_total, keys_max, stream, &x);
 }

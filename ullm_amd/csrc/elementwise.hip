@@ -435,6 +435,69 @@ extern "C" int ullm_silu_mul(const void* gu, void* out, int T_, int I, int dtype
   ULLM_LAUNCH_CHECK();
 }
 
+// ------------------------------------------------------------------ clamped gated activation
+// out = g' * sigmoid(alpha * g') * (u' + 1) with g' = min(gate, limit), u' = clamp(up, -limit, limit), for rows
+// gate | up [T, 2 I]: the gated unit of feed-forwards that bound both halves before they meet.
+template <typename T>
+__device__ __forceinline__ float clamped_glu(float g, float u, float limit, float alpha) {
+  g = fminf(g, limit);
+  u = fminf(fmaxf(u, -limit), limit);
+  // 32-bit mode: exact exponential and division; bfloat16: the hardware's, then rounded
+  const float sg = sizeof(T) == 4 ? 1.f / (1.f + expf(-alpha * g))
+                                  : __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-1.4426950408889634f * alpha * g));
+  return g * sg * (u + 1.f);
+}
+template <typename T>
+__global__ void glu_clamped_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t total, float limit,
+                                   float alpha) {
+  size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const size_t t = idx / I;
+  const int i = (int)(idx - t * I);
+  const T* row = gu + t * (size_t)(2 * I);
+  st_f32(out + idx, clamped_glu<T>(ld_f32(row + i), ld_f32(row + I + i), limit, alpha));
+}
+template <typename T>
+__global__ void glu_clamped_vec_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t total4, float limit,
+                                       float alpha) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;    // group of 4 consecutive outputs
+  if (idx >= total4) return;
+  const size_t per_row = (size_t)(I / 4);
+  const size_t t = idx / per_row;
+  const int i = 4 * (int)(idx - t * per_row);
+  const T* row = gu + t * (size_t)(2 * I);
+  const float4 g = ld4_f32_stream(row + i), u = ld4_f32_stream(row + I + i);
+  st4_f32(out + t * (size_t)I + i,
+          make_float4(clamped_glu<T>(g.x, u.x, limit, alpha), clamped_glu<T>(g.y, u.y, limit, alpha),
+                      clamped_glu<T>(g.z, u.z, limit, alpha), clamped_glu<T>(g.w, u.w, limit, alpha)));
+}
+
+extern "C" int ullm_glu_clamped(const void* gu, void* out, int T_, int I, float limit, float alpha, int dtype,
+                                hipStream_t stream) {
+  if (T_ <= 0) return 0;
+  if (I <= 0 || !(limit > 0.f)) return ULLM_ERR_SHAPE;
+  const size_t total = (size_t)T_ * I;
+  if (I % 4 == 0 && !(((uintptr_t)gu | (uintptr_t)out) & 15)) {
+    const size_t total4 = total / 4;
+    dim3 vblock(256), vgrid((unsigned)((total4 + 255) / 256));
+    if (dtype == ULLM_F32)
+      hipLaunchKernelGGL(glu_clamped_vec_kernel<float>, vgrid, vblock, 0, stream, (const float*)gu, (float*)out, I, total4, limit, alpha);
+    else if (dtype == ULLM_BF16)
+      hipLaunchKernelGGL(glu_clamped_vec_kernel<bf16_t>, vgrid, vblock, 0, stream, (const bf16_t*)gu, (bf16_t*)out, I, total4, limit, alpha);
+    else
+      return ULLM_ERR_DTYPE;
+    ULLM_LAUNCH_CHECK();
+  }
+  dim3 block(256), grid((unsigned)((total + 255) / 256));
+  if (dtype == ULLM_F32)
+    hipLaunchKernelGGL(glu_clamped_kernel<float>, grid, block, 0, stream, (const float*)gu, (float*)out, I, total, limit, alpha);
+  else if (dtype == ULLM_BF16)
+    hipLaunchKernelGGL(glu_clamped_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)gu, (bf16_t*)out, I, total, limit, alpha);
+  else
+    return ULLM_ERR_DTYPE;
+  ULLM_LAUNCH_CHECK();
+}
+
 // ------------------------------------------------------------------ stacks of partial sums to one result
 // out[m][n] = sum over s of stacks[s][m][n] (+ bias[n]), the stacks added in order, four columns a thread.
 // What a first projection needs from the partial-sums product (the last projections' stacks are added by
@@ -478,7 +541,8 @@ extern "C" int ullm_sum_stacks(const float* stacks, int n_stacks, const float* b
 // One wave per (token, head) of the fused projection row  [q heads | k heads | v heads].
 //   q heads: per-head RMS norm (gain shared by all heads, may be null), rotation, written to q_out
 //   k heads: the same with the k gain, written into the token's cache page
-//   v heads: copied into the cache page
+//   v heads: copied into the cache page; value head j is head v_head0 + j of the row (nq + nkv where the
+//            row holds values of its own; nq where the values are the keys as projected, before norm and rotation)
 // Rotation: pair (i, i + rot/2) for style 1 (half split), (2i, 2i+1) for style 2, i < rot/2;
 //   o_a = a cos - b sin, o_b = b cos + a sin with cos/sin = table[pos, i], table[pos, rot/2 + i];
 //   dims >= rot pass through.  style 0: no rotation.
@@ -494,12 +558,12 @@ __global__ void qk_norm_rope_write_kernel(
     const float* __restrict__ cos_sin, int table_rows, int rot, int style,
     const int* __restrict__ positions, const int* __restrict__ token_entry,
     const int* __restrict__ block_table, int bt_stride, T* __restrict__ k_pool, T* __restrict__ v_pool,
-    int page_size, int nq, int nkv, int hd, int write_kv) {
+    int page_size, int nq, int nkv, int hd, int write_kv, int v_head0) {
   __shared__ float vals[MAX_HEAD_DIM];
   const int t = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   const int pos = positions[t];
-  const T* src = qkv + (size_t)t * qkv_stride + (size_t)head * hd;
   const bool is_q = head < nq, is_k = !is_q && head < nq + nkv;
+  const T* src = qkv + (size_t)t * qkv_stride + (size_t)(is_q || is_k ? head : v_head0 + head - nq - nkv) * hd;
   T* dst;
   if (is_q) {
     dst = q_out + (size_t)t * q_out_stride + (size_t)head * hd;
@@ -555,7 +619,7 @@ __global__ void qk_norm_rope_write_kernel(
 template <typename T>
 __device__ __forceinline__ void value_runs_block(
     const T* __restrict__ qkv, int qkv_stride, const int* __restrict__ positions, const int* __restrict__ token_entry,
-    const int* __restrict__ block_table, int bt_stride, T* __restrict__ v_pool, int page_size, int nq, int nkv,
+    const int* __restrict__ block_table, int bt_stride, T* __restrict__ v_pool, int page_size, int v_head0, int nkv,
     int hd, int n_tokens, int block) {
   __shared__ __attribute__((aligned(16))) T tile[VALUE_RUN_TOKENS * VALUE_RUN_MAX_HD];
   __shared__ int s_page[VALUE_RUN_TOKENS], s_off[VALUE_RUN_TOKENS], s_run[VALUE_RUN_TOKENS];
@@ -566,7 +630,7 @@ __device__ __forceinline__ void value_runs_block(
   for (int c = threadIdx.x; c < n * pieces; c += blockDim.x) {
     const int tok = c / pieces, part = c % pieces;
     *reinterpret_cast<uint4*>(tile + tok * hd + part * PER16) = *reinterpret_cast<const uint4*>(
-        qkv + (size_t)(tok0 + tok) * qkv_stride + (size_t)(nq + nkv + kvh) * hd + part * PER16);
+        qkv + (size_t)(tok0 + tok) * qkv_stride + (size_t)(v_head0 + kvh) * hd + part * PER16);
   }
   if ((int)threadIdx.x < n) {
     // a token leads a run if it is the block's first or does not continue its predecessor's group of 8
@@ -620,9 +684,10 @@ qk_norm_rope_write_vec_kernel(
     const float* __restrict__ cos_sin, int table_rows, int rot, int style,
     const int* __restrict__ positions, const int* __restrict__ token_entry,
     const int* __restrict__ block_table, int bt_stride, T* __restrict__ k_pool, T* __restrict__ v_pool,
-    int page_size, int nq, int nkv, int hd, int write_kv, int n_tokens, int blocks_per_token, int heads_per_thread) {
+    int page_size, int nq, int nkv, int hd, int write_kv, int n_tokens, int blocks_per_token, int heads_per_thread,
+    int v_head0) {
   if (blockIdx.x >= (unsigned)(n_tokens * blocks_per_token)) {
-    value_runs_block<T>(qkv, qkv_stride, positions, token_entry, block_table, bt_stride, v_pool, page_size, nq, nkv,
+    value_runs_block<T>(qkv, qkv_stride, positions, token_entry, block_table, bt_stride, v_pool, page_size, v_head0, nkv,
                         hd, n_tokens, (int)blockIdx.x - n_tokens * blocks_per_token);
     return;
   }
@@ -654,7 +719,7 @@ qk_norm_rope_write_vec_kernel(
     const bool is_q = head < nq, is_k = !is_q && head < nq + nkv;
     float x[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     if (live) {
-      const T* src = qkv + (size_t)t * qkv_stride + (size_t)head * hd + d0;
+      const T* src = qkv + (size_t)t * qkv_stride + (size_t)(is_q || is_k ? head : v_head0 + head - nq - nkv) * hd + d0;
       const float4 lo = ld4_f32_stream(src), hi = ld4_f32_stream(src + 4);     // the projection row is read once
       x[0] = lo.x; x[1] = lo.y; x[2] = lo.z; x[3] = lo.w; x[4] = hi.x; x[5] = hi.y; x[6] = hi.z; x[7] = hi.w;
     }
@@ -727,9 +792,10 @@ extern "C" int ullm_qk_norm_rope_write(
     const float* k_gain, float eps, const float* cos_sin, int table_rows, int rot, int style,
     const int* positions, const int* token_entry, const int* block_table, int bt_stride,
     void* k_pool, void* v_pool, int page_size, int T_, int nq, int nkv, int hd, int write_kv,
-    int dtype, hipStream_t stream) {
+    int v_head0, int dtype, hipStream_t stream) {
   if (T_ <= 0) return 0;
   if (hd <= 0 || hd > MAX_HEAD_DIM || nq <= 0 || nkv <= 0 || page_size <= 0) return ULLM_ERR_SHAPE;
+  if (v_head0 != nq + nkv && v_head0 != nq) return ULLM_ERR_SHAPE;
   if (rot < 0 || rot > hd || (rot & 1) || (style != 0 && style != 1 && style != 2)) return ULLM_ERR_SHAPE;
   if (style != 0 && rot > 0 && (!cos_sin || table_rows <= 0)) return ULLM_ERR_SHAPE;
   const int lph = hd / 8;
@@ -759,7 +825,7 @@ extern "C" int ullm_qk_norm_rope_write(
 #define GOV(TT) hipLaunchKernelGGL(qk_norm_rope_write_vec_kernel<TT>, vgrid, vblock, 0, stream, \
     (const TT*)qkv, qkv_stride, (TT*)q_out, q_out_stride, q_gain, k_gain, eps, cos_sin, table_rows, \
     rot, style, positions, token_entry, block_table, bt_stride, (TT*)k_pool, (TT*)v_pool, page_size, \
-    nq, nkv, hd, kv_flags, T_, blocks_per_token, heads_per_thread)
+    nq, nkv, hd, kv_flags, T_, blocks_per_token, heads_per_thread, v_head0)
     if (dtype == ULLM_F32) GOV(float);
     else if (dtype == ULLM_BF16) GOV(bf16_t);
     else return ULLM_ERR_DTYPE;
@@ -770,7 +836,7 @@ extern "C" int ullm_qk_norm_rope_write(
 #define GO(TT) hipLaunchKernelGGL(qk_norm_rope_write_kernel<TT>, grid, block, 0, stream, \
     (const TT*)qkv, qkv_stride, (TT*)q_out, q_out_stride, q_gain, k_gain, eps, cos_sin, table_rows, \
     rot, style, positions, token_entry, block_table, bt_stride, (TT*)k_pool, (TT*)v_pool, page_size, \
-    nq, nkv, hd, write_kv)
+    nq, nkv, hd, write_kv, v_head0)
   if (dtype == ULLM_F32) GO(float);
   else if (dtype == ULLM_BF16) GO(bf16_t);
   else return ULLM_ERR_DTYPE;

@@ -79,6 +79,7 @@ extern "C" int ullm_gemm_simple(const void* A, int lda, const void* W, int ldw, 
     case 7: GO(bf16_t, bf16_t, bf16_t); break;
     case 6: GO(bf16_t, bf16_t, float); break;
     case 2: GO(float, bf16_t, float); break;
+    case 4: GO(bf16_t, float, float); break;     // 32-bit weights on rounded activations (a router)
     default: return ULLM_ERR_DTYPE;
   }
 #undef GO

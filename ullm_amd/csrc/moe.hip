@@ -1,0 +1,385 @@
+// Routed feed-forward (mixture of experts): routing, the grouping of (token, chosen expert) pairs by expert,
+// the experts' two products over the grouped rows, and the weighted sum.  Nothing here waits for the device
+// or sizes a launch by values: grids are made for the most tiles any routing can give, and a block whose
+// tile is empty leaves at once, so a step can be captured into a graph.
+//
+//   route     logits [T, R] (R = experts with weights + identity experts) -> softmax over all R, the choice by
+//             softmax + correction, the `top` largest (ties: the lower index), weights = the chosen experts'
+//             softmax values over their sum (+ 1e-20).  All 32-bit.  One wave per token.
+//   sort      pairs (token, k) -> rows ("slots") grouped by expert; identity experts (index >= experts) get no
+//             slot.  Which slot inside its expert a pair gets depends on timing; no value does: every row of a
+//             product is a function of that row alone.  Also the tile list: (expert, first slot, rows <= tile_rows).
+//   gate_up   act[slot, :] = glu(x[token of slot] Wg[e]^T, x Wu[e]^T) with the clamped gated unit
+//             g' = min(g, limit), u' = clamp(u, -limit, limit), act = g' sigmoid(alpha g') (u' + 1)
+//   down      y[slot, :] = act[slot] Wd[e]^T, 32-bit
+//   combine   out[t] = base[t] + bias + shared[t] + sum_k weight[t, k] * (expert k has weights ? y[slot(t, k)] : x[t]),
+//             added in the order of k, 32-bit.
+//
+// Products: bfloat16 on v_mfma_f32_16x16x32_bf16 (A operand = 16 rows of an expert's matrix, lane (r, g) holds
+// W[n0 + r][k + 8g .. +8]; B operand = 16 grouped rows of x; lane (r, g) then holds out[row r][column n0 + 4g .. +4]),
+// or for float32 and for shapes the tiles do not take a kernel with one wave per output value that sums K in a
+// fixed order.  Expert matrices are stacked: gate|up [experts, 2 ff, hidden], down [experts, hidden, ff].
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+union Pack8 {
+  bf16x8_t v;
+  uint4 u4;
+};
+
+#define MOE_MAX_ROUTER 1024          // router outputs (experts + identity experts)
+#define MOE_MAX_TOP 32
+
+// ------------------------------------------------------------------------------- routing
+__global__ void __launch_bounds__(64)
+moe_route_kernel(const float* __restrict__ logits, int ld, const float* __restrict__ correction, int n_router, int top,
+                 int* __restrict__ ids, float* __restrict__ weights) {
+  __shared__ float s_soft[MOE_MAX_ROUTER], s_choice[MOE_MAX_ROUTER];
+  __shared__ float s_pick[MOE_MAX_TOP];
+  const int t = blockIdx.x, lane = threadIdx.x;
+  const float* z = logits + (size_t)t * ld;
+  float mx = -INFINITY;
+  for (int e = lane; e < n_router; e += 64) mx = fmaxf(mx, z[e]);
+  mx = wave_max(mx);
+  float sum = 0.f;
+  for (int e = lane; e < n_router; e += 64) {
+    const float p = expf(z[e] - mx);
+    s_soft[e] = p;
+    sum += p;
+  }
+  sum = wave_sum(sum);
+  for (int e = lane; e < n_router; e += 64) {
+    const float s = s_soft[e] / sum;
+    s_soft[e] = s;
+    s_choice[e] = s + (correction ? correction[e] : 0.f);
+  }
+  __syncthreads();
+  float total = 0.f;
+  for (int k = 0; k < top; ++k) {
+    float best = -INFINITY;
+    int at = 0x7fffffff;
+    for (int e = lane; e < n_router; e += 64) {
+      const float c = s_choice[e];
+      if (c > best || (c == best && e < at)) {
+        best = c;
+        at = e;
+      }
+    }
+#pragma unroll
+    for (int m = 32; m > 0; m >>= 1) {
+      const float ob = __shfl_xor(best, m, 64);
+      const int oa = __shfl_xor(at, m, 64);
+      if (ob > best || (ob == best && oa < at)) {
+        best = ob;
+        at = oa;
+      }
+    }
+    if (at >= n_router) at = k < n_router ? k : 0;       // every value a NaN: any expert
+    const float s = s_soft[at];
+    total += s;
+    if (lane == 0) {
+      ids[(size_t)t * top + k] = at;
+      s_pick[k] = s;
+      s_choice[at] = -INFINITY;
+    }
+    __syncthreads();
+  }
+  if (lane < top) weights[(size_t)t * top + lane] = s_pick[lane] / (total + 1e-20f);
+}
+
+extern "C" int ullm_moe_route(const float* logits, int ld, const float* correction, int T_, int n_router, int top,
+                              int* ids, float* weights, hipStream_t stream) {
+  if (T_ <= 0) return 0;
+  if (n_router < 1 || n_router > MOE_MAX_ROUTER || top < 1 || top > MOE_MAX_TOP || top > n_router || ld < n_router)
+    return ULLM_ERR_SHAPE;
+  hipLaunchKernelGGL(moe_route_kernel, dim3(T_), dim3(64), 0, stream, logits, ld, correction, n_router, top, ids, weights);
+  ULLM_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------------------------------------- grouping by expert
+// One block.  offsets [experts + 1]; slot_of_pair [pairs] (-1: the pair's expert has no weights); token_of_slot [pairs];
+// tiles [max_tiles][3] = (expert, first slot, rows), rows 0 for the tiles no expert filled.
+__global__ void __launch_bounds__(1024)
+moe_sort_kernel(const int* __restrict__ ids, int n_pairs, int top, int n_experts, int tile_rows,
+                int* __restrict__ offsets, int* __restrict__ slot_of_pair, int* __restrict__ token_of_slot,
+                int* __restrict__ tiles, int max_tiles) {
+  __shared__ int count[MOE_MAX_ROUTER], start[MOE_MAX_ROUTER + 1], cursor[MOE_MAX_ROUTER], tile_base[MOE_MAX_ROUTER + 1];
+  const int tid = threadIdx.x;
+  for (int e = tid; e < n_experts; e += blockDim.x) count[e] = 0;
+  __syncthreads();
+  for (int p = tid; p < n_pairs; p += blockDim.x) {
+    const int e = ids[p];
+    if (e >= 0 && e < n_experts) atomicAdd(&count[e], 1);
+  }
+  __syncthreads();
+  if (tid == 0) {
+    int off = 0, tb = 0;
+    for (int e = 0; e < n_experts; ++e) {
+      start[e] = off;
+      cursor[e] = off;
+      tile_base[e] = tb;
+      off += count[e];
+      tb += (count[e] + tile_rows - 1) / tile_rows;
+    }
+    start[n_experts] = off;
+    tile_base[n_experts] = tb;
+  }
+  __syncthreads();
+  for (int e = tid; e <= n_experts; e += blockDim.x) offsets[e] = start[e];
+  for (int p = tid; p < n_pairs; p += blockDim.x) {
+    const int e = ids[p];
+    int slot = -1;
+    if (e >= 0 && e < n_experts) {
+      slot = atomicAdd(&cursor[e], 1);
+      token_of_slot[slot] = p / top;
+    }
+    slot_of_pair[p] = slot;
+  }
+  for (int e = tid; e < n_experts; e += blockDim.x) {
+    const int first = tile_base[e], n = tile_base[e + 1] - first;
+    for (int i = 0; i < n && first + i < max_tiles; ++i) {
+      const int left = count[e] - i * tile_rows;
+      tiles[3 * (first + i)] = e;
+      tiles[3 * (first + i) + 1] = start[e] + i * tile_rows;
+      tiles[3 * (first + i) + 2] = left < tile_rows ? left : tile_rows;
+    }
+  }
+  for (int i = tile_base[n_experts] + tid; i < max_tiles; i += blockDim.x) {
+    tiles[3 * i] = 0;
+    tiles[3 * i + 1] = 0;
+    tiles[3 * i + 2] = 0;
+  }
+}
+
+extern "C" int ullm_moe_sort(const int* ids, int n_pairs, int top, int n_experts, int tile_rows, int* offsets,
+                             int* slot_of_pair, int* token_of_slot, int* tiles, int max_tiles, hipStream_t stream) {
+  if (n_pairs <= 0) return 0;
+  if (n_experts < 1 || n_experts > MOE_MAX_ROUTER || top < 1 || tile_rows < 1 || max_tiles < 1) return ULLM_ERR_SHAPE;
+  // every routing fits: sum over experts of ceil(count / tile_rows) <= pairs / tile_rows + experts in use
+  const long long most = (long long)n_pairs / tile_rows + (n_experts < n_pairs ? n_experts : n_pairs);
+  if (max_tiles < most) return ULLM_ERR_SHAPE;
+  hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, stream, ids, n_pairs, top, n_experts, tile_rows, offsets,
+                     slot_of_pair, token_of_slot, tiles, max_tiles);
+  ULLM_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------------------------------------- the clamped gated unit
+template <bool EXACT>
+__device__ __forceinline__ float moe_glu(float g, float u, float limit, float alpha) {
+  g = fminf(g, limit);
+  u = fminf(fmaxf(u, -limit), limit);
+  const float sg = EXACT ? 1.f / (1.f + expf(-alpha * g))
+                         : __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-1.4426950408889634f * alpha * g));
+  return g * sg * (u + 1.f);
+}
+
+// ------------------------------------------------------------------------------- products, one wave per value
+// grid (tiles, column blocks); a block of 4 waves takes one tile's rows in turn, the row of x in shared memory,
+// and each wave its share of the block's columns: lanes stride K, then the wave adds up (a fixed order).
+template <typename T, bool GATED>
+__global__ void __launch_bounds__(256)
+moe_rows_simple_kernel(const T* __restrict__ x, int ldx, const int* __restrict__ row_index,
+                       const T* __restrict__ w, const int* __restrict__ tiles, void* __restrict__ out_, int ldo,
+                       int n_out, int K, int cols_per_block, float limit, float alpha) {
+  extern __shared__ float xrow[];
+  const int tile = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int e = tiles[3 * tile], slot0 = tiles[3 * tile + 1], rows = tiles[3 * tile + 2];
+  if (rows <= 0) return;
+  const int c0 = blockIdx.y * cols_per_block;
+  const int c1 = c0 + cols_per_block < n_out ? c0 + cols_per_block : n_out;
+  const size_t w_rows = GATED ? 2 * (size_t)n_out : (size_t)n_out;
+  const T* we = w + (size_t)e * w_rows * K;
+  for (int r = 0; r < rows; ++r) {
+    const int slot = slot0 + r;
+    const T* xr = x + (size_t)(row_index ? row_index[slot] : slot) * ldx;
+    __syncthreads();
+    for (int i = tid; i < K; i += 256) xrow[i] = ld_f32(xr + i);
+    __syncthreads();
+    for (int c = c0 + wave; c < c1; c += 4) {
+      const T* wg = we + (size_t)c * K;
+      float a = 0.f, b = 0.f;
+      for (int i = lane; i < K; i += 64) {
+        a = fmaf(xrow[i], ld_f32(wg + i), a);
+        if (GATED) b = fmaf(xrow[i], ld_f32(wg + (size_t)n_out * K + i), b);
+      }
+      a = wave_sum(a);
+      if (GATED) b = wave_sum(b);
+      if (lane == 0) {
+        if (GATED) st_f32(reinterpret_cast<T*>(out_) + (size_t)slot * ldo + c, moe_glu<sizeof(T) == 4>(a, b, limit, alpha));
+        else reinterpret_cast<float*>(out_)[(size_t)slot * ldo + c] = a;
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------- products on the matrix cores
+// grid (tiles, column blocks); tile = up to 16 * MT grouped rows of one expert; a block's WAVES waves take 16
+// output columns each (GATED: the 16 gate rows and the 16 up rows of those columns) over all of K, two steps of 32
+// in flight.  No load stands under a condition: a row past the tile's reads its last row, a column past the end
+// the last column, a piece past the end of K the row's last piece (and is replaced by zeros); none is stored.
+template <int MT, bool GATED>
+__global__ void __launch_bounds__(256)
+moe_rows_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const int* __restrict__ row_index,
+                     const bf16_t* __restrict__ w, const int* __restrict__ tiles, void* __restrict__ out_, int ldo,
+                     int n_out, int K, float limit, float alpha) {
+  const int tile = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 15, g = lane >> 4;
+  const int e = tiles[3 * tile], slot0 = tiles[3 * tile + 1], rows = tiles[3 * tile + 2];
+  if (rows <= 0) return;
+  const int n0 = (blockIdx.y * 4 + wave) * 16;
+  if (n0 >= n_out) return;
+  const size_t w_rows = GATED ? 2 * (size_t)n_out : (size_t)n_out;
+  const int wrow = n0 + r < n_out ? n0 + r : n_out - 1;
+  const bf16_t* wg = w + ((size_t)e * w_rows + wrow) * K;
+  const bf16_t* wu = wg + (size_t)n_out * K;
+  const bf16_t* xr[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    const int row = 16 * t + r < rows ? 16 * t + r : rows - 1;
+    xr[t] = x + (size_t)(row_index ? row_index[slot0 + row] : slot0 + row) * ldx;
+  }
+  f32x4_t acc_g[MT], acc_u[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    acc_g[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    acc_u[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  }
+  const int last_piece = K - 8;                          // K is a multiple of 8
+  const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+  for (int k0 = 0; k0 < K; k0 += 64) {
+    Pack8 a_g[2], a_u[2], b[2][MT];
+    bool in[2];
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      const int k = k0 + 32 * s + 8 * g;
+      in[s] = k <= last_piece;
+      const int kk = in[s] ? k : last_piece;
+      a_g[s].u4 = ld_stream16(wg + kk);
+      if (GATED) a_u[s].u4 = ld_stream16(wu + kk);
+#pragma unroll
+      for (int t = 0; t < MT; ++t) b[s][t].u4 = ld16(xr[t] + kk);
+    }
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        if (!in[s]) b[s][t].u4 = zero;
+        acc_g[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_g[s].v, b[s][t].v, acc_g[t], 0, 0, 0);
+        if (GATED) acc_u[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_u[s].v, b[s][t].v, acc_u[t], 0, 0, 0);
+      }
+    }
+  }
+  // lane (r, g): row r of each 16-row group, columns n0 + 4g .. + 4
+  const int c = n0 + 4 * g;
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    const int row = 16 * t + r;
+    if (row >= rows) continue;
+    const size_t at = (size_t)(slot0 + row) * ldo + c;
+    if (GATED) {
+      bf16_t* o = reinterpret_cast<bf16_t*>(out_) + at;
+      float v[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = moe_glu<false>(acc_g[t][i], acc_u[t][i], limit, alpha);
+      if (c + 3 < n_out && (ldo & 3) == 0) {
+        *reinterpret_cast<uint2*>(o) = make_uint2(pack2_bf16(v[0], v[1]), pack2_bf16(v[2], v[3]));
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (c + i < n_out) o[i] = f32_to_bf16_bits(v[i]);
+      }
+    } else {
+      float* o = reinterpret_cast<float*>(out_) + at;
+      if (c + 3 < n_out && (ldo & 3) == 0) {
+        *reinterpret_cast<float4*>(o) = make_float4(acc_g[t][0], acc_g[t][1], acc_g[t][2], acc_g[t][3]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (c + i < n_out) o[i] = acc_g[t][i];
+      }
+    }
+  }
+}
+
+// Rows of a tile the matrix-core kernels take for a launch made with `tile_rows` rows a tile.
+extern "C" int ullm_moe_mfma_supports(int K, int ldx, int tile_rows) {
+  return K >= 8 && K % 8 == 0 && ldx % 8 == 0 && (tile_rows == 16 || tile_rows == 32 || tile_rows == 64);
+}
+
+// out[slot] = glu(x[row_index[slot]] Wg^T, x Wu^T) (gated: out in x's dtype, w [experts, 2 n_out, K]) or
+// x[slot] W^T (not gated: out float32, w [experts, n_out, K]) over the tiles' rows.  row_index may be null.
+extern "C" int ullm_moe_rows(const void* x, int ldx, const int* row_index, const void* w, const int* tiles,
+                             int max_tiles, int tile_rows, void* out, int ldo, int n_out, int K, int gated,
+                             float limit, float alpha, int dtype, hipStream_t stream) {
+  if (max_tiles <= 0) return 0;
+  if (n_out < 1 || K < 1 || ldx < K || ldo < n_out || tile_rows < 1) return ULLM_ERR_SHAPE;
+  if (dtype == ULLM_BF16 && ullm_moe_mfma_supports(K, ldx, tile_rows) && !((uintptr_t)x & 15) && !((uintptr_t)w & 15)) {
+    dim3 grid(max_tiles, (n_out + 63) / 64), block(256);
+    if (grid.y > 65535) return ULLM_ERR_SHAPE;
+#define GO(MT, G) hipLaunchKernelGGL((moe_rows_mfma_kernel<MT, G>), grid, block, 0, stream, (const bf16_t*)x, ldx, row_index, \
+    (const bf16_t*)w, tiles, out, ldo, n_out, K, limit, alpha)
+    if (tile_rows == 16) { if (gated) GO(1, true); else GO(1, false); }
+    else if (tile_rows == 32) { if (gated) GO(2, true); else GO(2, false); }
+    else { if (gated) GO(4, true); else GO(4, false); }
+#undef GO
+    ULLM_LAUNCH_CHECK();
+  }
+  if ((size_t)K * sizeof(float) > 64 * 1024) return ULLM_ERR_SHAPE;
+  const int cols_per_block = 64;
+  dim3 grid(max_tiles, (n_out + cols_per_block - 1) / cols_per_block), block(256);
+  if (grid.y > 65535) return ULLM_ERR_SHAPE;
+  const size_t lds = (size_t)K * sizeof(float);
+#define GO(TT, G) hipLaunchKernelGGL((moe_rows_simple_kernel<TT, G>), grid, block, lds, stream, (const TT*)x, ldx, row_index, \
+    (const TT*)w, tiles, out, ldo, n_out, K, cols_per_block, limit, alpha)
+  if (dtype == ULLM_F32) { if (gated) GO(float, true); else GO(float, false); }
+  else if (dtype == ULLM_BF16) { if (gated) GO(bf16_t, true); else GO(bf16_t, false); }
+  else return ULLM_ERR_DTYPE;
+#undef GO
+  ULLM_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------------------------------------- the weighted sum
+// out[t][c] = base[t][c] + bias[c] + shared[t][c] + sum_k weights[t][k] * (ids[t][k] < n_experts ? y[slot][c] : x[t][c]);
+// base (float32 or TX), bias (float32), shared (TX) may be null.  Four columns a thread where rows allow.
+template <typename TX, typename TB>
+__global__ void __launch_bounds__(256)
+moe_combine_kernel(const float* __restrict__ y, const TX* __restrict__ x, int ldx, const int* __restrict__ ids,
+                   const float* __restrict__ weights, const int* __restrict__ slot_of_pair, int top, int n_experts,
+                   const TB* __restrict__ base, const float* __restrict__ bias, const TX* __restrict__ shared,
+                   float* __restrict__ out, int H) {
+  const int t = blockIdx.x;
+  for (int c = threadIdx.x; c < H; c += 256) {
+    float a = base ? ld_f32(base + (size_t)t * H + c) : 0.f;
+    if (bias) a += bias[c];
+    if (shared) a += ld_f32(shared + (size_t)t * H + c);
+    for (int k = 0; k < top; ++k) {
+      const int e = ids[(size_t)t * top + k];
+      const float wk = weights[(size_t)t * top + k];
+      const float v = e < n_experts ? y[(size_t)slot_of_pair[(size_t)t * top + k] * H + c] : ld_f32(x + (size_t)t * ldx + c);
+      a = fmaf(wk, v, a);
+    }
+    out[(size_t)t * H + c] = a;
+  }
+}
+
+extern "C" int ullm_moe_combine(const float* y, const void* x, int ldx, const int* ids, const float* weights,
+                                const int* slot_of_pair, int top, int n_experts, const void* base, int base_dtype,
+                                const float* bias, const void* shared, float* out, int T_, int H, int dtype,
+                                hipStream_t stream) {
+  if (T_ <= 0) return 0;
+  if (H < 1 || top < 1 || ldx < H) return ULLM_ERR_SHAPE;
+  dim3 grid(T_), block(256);
+#define GO(TX, TB) hipLaunchKernelGGL((moe_combine_kernel<TX, TB>), grid, block, 0, stream, y, (const TX*)x, ldx, ids, weights, \
+    slot_of_pair, top, n_experts, (const TB*)base, bias, (const TX*)shared, out, H)
+  if (dtype == ULLM_F32) {
+    if (base && base_dtype != ULLM_F32) return ULLM_ERR_DTYPE;
+    GO(float, float);
+  } else if (dtype == ULLM_BF16) {
+    if (base && base_dtype == ULLM_BF16) GO(bf16_t, bf16_t);
+    else GO(bf16_t, float);
+  } else {
+    return ULLM_ERR_DTYPE;
+  }
+#undef GO
+  ULLM_LAUNCH_CHECK();
+}

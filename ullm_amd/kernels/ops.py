@@ -209,6 +209,20 @@ def silu_mul(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch
     return out
 
 
+def glu_clamped(gate_up: torch.Tensor, limit: float, alpha: float, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """g * sigmoid(alpha * g) * (u + 1) with g = min(gate, limit), u = clamp(up, -limit, limit), for a contiguous
+    [T, 2I] input gate | up."""
+    T, two_i = gate_up.shape
+    _need(two_i % 2 == 0 and gate_up.is_contiguous(), "gate_up must be contiguous [T, 2I]")
+    inter = two_i // 2
+    if out is None:
+        out = torch.empty((T, inter), dtype=gate_up.dtype, device=gate_up.device)
+    _need(out.shape == (T, inter) and out.is_contiguous() and out.dtype == gate_up.dtype, "bad glu_clamped output")
+    _check(build.load("elementwise").ullm_glu_clamped(_p(gate_up), _p(out), _c_int(T), _c_int(inter), _c_float(limit),
+                                                      _c_float(alpha), _c_int(_dt(gate_up)), _stream()), "glu_clamped")
+    return out
+
+
 def sum_stacks(stacks: torch.Tensor, bias: Optional[torch.Tensor] = None,
                out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
     """The sum over the first dimension of float32 ``stacks`` [S, M, N] (what :func:`gemm_partial_sums` leaves), added
@@ -229,13 +243,16 @@ def qk_norm_rope_write(qkv: torch.Tensor, q_out: torch.Tensor, q_gain: Optional[
                        k_gain: Optional[torch.Tensor], eps: float, cos_sin: Optional[torch.Tensor],
                        rotary_dim: int, style: int, positions: torch.Tensor, token_entry: torch.Tensor,
                        block_table: torch.Tensor, k_pool: Optional[torch.Tensor], v_pool: Optional[torch.Tensor],
-                       page_size: int, nq: int, nkv: int, hd: int, write_kv: bool) -> None:
+                       page_size: int, nq: int, nkv: int, hd: int, write_kv: bool,
+                       values_from_keys: bool = False) -> None:
     """Per-head norm and rotation of q (to ``q_out`` [T, nq*hd]) and k, and the cache write of k and v.
     ``qkv`` is [T, (nq + 2 nkv) * hd]; key pool [pages, nkv, page_size, hd], value pool
     [pages, nkv, hd, page_size]; ``block_table`` is
-    int32 [B, stride] with one row per batch entry."""
+    int32 [B, stride] with one row per batch entry.  With ``values_from_keys`` the row is [T, (nq + nkv) * hd]
+    and the values written are the keys as projected, before norm and rotation."""
     T = qkv.shape[0]
-    _need(qkv.dim() == 2 and qkv.shape[1] == (nq + 2 * nkv) * hd and qkv.stride(1) == 1, "bad qkv shape")
+    _need(qkv.dim() == 2 and qkv.shape[1] == (nq + (1 if values_from_keys else 2) * nkv) * hd and qkv.stride(1) == 1,
+          "bad qkv shape")
     _need(q_out.shape == (T, nq * hd) and q_out.is_contiguous() and q_out.dtype == qkv.dtype, "bad q_out")
     _need(hd <= 512, f"head_dim {hd} exceeds 512")
     _i32(positions, "positions", T)
@@ -259,7 +276,7 @@ def qk_norm_rope_write(qkv: torch.Tensor, q_out: torch.Tensor, q_gain: Optional[
         _c_float(eps), _p(cos_sin), _c_int(table_rows), _c_int(rotary_dim), _c_int(style), _p(positions),
         _p(token_entry), _p(block_table), _c_int(block_table.stride(0)), _p(k_pool), _p(v_pool),
         _c_int(page_size), _c_int(T), _c_int(nq), _c_int(nkv), _c_int(hd), _c_int(1 if write_kv else 0),
-        _c_int(_dt(qkv)), _stream()), "qk_norm_rope_write")
+        _c_int(nq if values_from_keys else nq + nkv), _c_int(_dt(qkv)), _stream()), "qk_norm_rope_write")
 
 
 
@@ -481,12 +498,21 @@ def _check_distance_bias(bias: Optional[torch.Tensor], nq: int) -> int:
     return bias.shape[1]
 
 
+def _check_sink(sink: Optional[torch.Tensor], nq: int) -> None:
+    if sink is not None:
+        _need(sink.dtype == torch.float32 and sink.numel() == nq and sink.is_contiguous(),
+              f"attention sinks must be contiguous float32 [{nq}]")
+
+
 def paged_attention_generic(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
                             positions: torch.Tensor, token_entry: torch.Tensor, block_table: torch.Tensor,
                             page_size: int, nq: int, nkv: int, hd: int, scale: float, window: int,
-                            out: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+                            out: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None,
+                            sink: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``bias`` (float32 [nq, rows]): bias[h, min(distance, rows - 1)] is added to the scaled score of a key
-    ``distance`` positions behind the query."""
+    ``distance`` positions behind the query.  ``sink`` (float32 [nq]): exp(sink[h]) is one more term of the
+    softmax's denominator, with no key and no value."""
+    _check_sink(sink, nq)
     T = q.shape[0]
     _need(q.shape == (T, nq * hd) and q.stride(1) == 1, "q must be [T, nq*hd]")
     _need(hd <= 512 and nq % nkv == 0, "head_dim > 512 or heads not a multiple of kv heads")
@@ -503,7 +529,7 @@ def paged_attention_generic(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch
         _p(q), _c_int(q.stride(0)), _p(out), _c_int(out.stride(0)), _p(k_pool), _p(v_pool), _p(positions),
         _p(token_entry), _p(block_table), _c_int(block_table.stride(0)), _c_int(page_size), _c_int(T),
         _c_int(nq), _c_int(nkv), _c_int(hd), _c_float(scale), _c_int(window), _p(bias),
-        _c_int(_check_distance_bias(bias, nq)), _c_int(_dt(q)), _stream()),
+        _c_int(_check_distance_bias(bias, nq)), _p(sink), _c_int(_dt(q)), _stream()),
         "paged_attention_generic")
     return out
 
@@ -816,11 +842,13 @@ def decode_split(n_items: int, nkv: int, groups: int, max_kv: int, hd: int = 128
 def attention_decode_mfma(q, out, k_pool, v_pool, token_list: Optional[torch.Tensor], n_items: int,
                           positions, token_entry, block_table, page_size: int, nq: int, nkv: int, hd: int,
                           scale: float, window: int, max_kv: int, splits: int = 0, waves: int = 0,
-                          bias_log2: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None) -> None:
+                          bias_log2: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
+                          sink_log2: Optional[torch.Tensor] = None) -> None:
     """One query token per item (``token_list`` int32 [n_items] names the tokens, None = tokens
     0..n_items-1) against its request's cache; with ``splits`` > 1 the keys go to several blocks whose
     partial results a second small kernel adds up.  ``bias_log2`` (float32 [nq, rows], a distance bias times
-    log2(e)) is added to the scores, ``gate`` (bfloat16 [T, >= nq]) gates every head's output by its sigmoid."""
+    log2(e)) is added to the scores, ``gate`` (bfloat16 [T, >= nq]) gates every head's output by its sigmoid,
+    ``sink_log2`` (float32 [nq], sinks times log2(e)) adds 2^sink to every head's sum of weights."""
     _check_pools(k_pool, v_pool, nkv, page_size, hd, torch.bfloat16)
     _need(q.dtype == torch.bfloat16 and q.stride(1) == 1 and q.shape[1] == nq * hd, "q must be bfloat16 [T, nq*hd]")
     _need(out.dtype == torch.bfloat16 and out.stride(1) == 1 and out.shape == q.shape, "bad attention output")
@@ -843,14 +871,15 @@ def attention_decode_mfma(q, out, k_pool, v_pool, token_list: Optional[torch.Ten
     ws = None
     if splits > 1:
         ws = torch.empty(n_items * nq * splits * (hd + 4), dtype=torch.float32, device=q.device)
-    if bias_log2 is not None or gate is not None:
+    if bias_log2 is not None or gate is not None or sink_log2 is not None:
         _check_gate(gate, q.shape[0], nq)
+        _check_sink(sink_log2, nq)
         _check(lib.ullm_attention_decode_extras(
             _p(q), _c_int(q.stride(0)), _p(out), _c_int(out.stride(0)), _p(k_pool), _p(v_pool), _p(token_list),
             _c_int(n_items), _p(positions), _p(token_entry), _p(block_table), _c_int(block_table.stride(0)),
             _c_int(page_size), _c_int(nq), _c_int(nkv), _c_int(hd), _c_float(scale), _c_int(window),
             _c_int(splits), _c_int(waves), _p(ws), _p(bias_log2), _c_int(_check_distance_bias(bias_log2, nq)), _p(gate),
-            _c_int(gate.stride(0) if gate is not None else 0), _stream()), "attention_decode_extras")
+            _c_int(gate.stride(0) if gate is not None else 0), _p(sink_log2), _stream()), "attention_decode_extras")
         return
     _check(lib.ullm_attention_decode(
         _p(q), _c_int(q.stride(0)), _p(out), _c_int(out.stride(0)), _p(k_pool), _p(v_pool), _p(token_list),
@@ -924,7 +953,8 @@ PREFILL_TILE = 32      # tokens of one request per prompt tile (two groups of 16
 def attention_prefill_mfma(q, out, k_pool, v_pool, tiles: torch.Tensor, n_tiles: int, positions, token_entry,
                            block_table, page_size: int, nq: int, nkv: int, hd: int, scale: float,
                            window: int, halves: int = 0, keys_total: int = 0, keys_max: int = 0,
-                           bias_log2: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None) -> None:
+                           bias_log2: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
+                           sink_log2: Optional[torch.Tensor] = None) -> None:
     """Tiles (first token, count <= PREFILL_TILE) of consecutive tokens of one request each, every
     token against the keys up to its own position.  ``halves``: 2 = two halves of a block share a
     tile's keys, 1 = one block takes them all, 0 = chosen from ``keys_total`` (the sum over the tiles of
@@ -939,15 +969,16 @@ def attention_prefill_mfma(q, out, k_pool, v_pool, tiles: torch.Tensor, n_tiles:
     _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.stride(1) == 1,
           "block_table must be int32 [B, stride]")
     lib = build.load("attention_mfma")
-    if bias_log2 is not None or gate is not None:
+    if bias_log2 is not None or gate is not None or sink_log2 is not None:
         _check_gate(gate, q.shape[0], nq)
+        _check_sink(sink_log2, nq)
         _check(lib.ullm_attention_prefill_extras(
             _p(q), _c_int(q.stride(0)), _p(out), _c_int(out.stride(0)), _p(k_pool), _p(v_pool), _p(tiles),
             _c_int(n_tiles), _p(positions), _p(token_entry), _p(block_table), _c_int(block_table.stride(0)),
             _c_int(page_size), _c_int(nq), _c_int(nkv), _c_int(hd), _c_float(scale), _c_int(window),
             _c_int(halves), ctypes.c_longlong(int(keys_total)), _c_int(keys_max), _p(bias_log2),
             _c_int(_check_distance_bias(bias_log2, nq)), _p(gate), _c_int(gate.stride(0) if gate is not None else 0),
-            _stream()), "attention_prefill_extras")
+            _p(sink_log2), _stream()), "attention_prefill_extras")
         return
     _check(lib.ullm_attention_prefill(
         _p(q), _c_int(q.stride(0)), _p(out), _c_int(out.stride(0)), _p(k_pool), _p(v_pool), _p(tiles),
@@ -978,7 +1009,8 @@ def _warn_general_attention(hd: int, page_size: int) -> None:
 def paged_attention(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, ctx, group, nq: int,
                     nkv: int, hd: int, scale: float, window: int, plan=None,
                     bias: Optional[torch.Tensor] = None, bias_log2: Optional[torch.Tensor] = None,
-                    gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+                    gate: Optional[torch.Tensor] = None, sink: Optional[torch.Tensor] = None,
+                    sink_log2: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention of the batch's queries over their requests' cached keys and values (the new
     tokens' rows included).  bfloat16 shapes the matrix-core kernels take go there (one launch for
     the one-token entries, one for the tiles of longer entries, both listed in ``plan``: arrays
@@ -986,27 +1018,135 @@ def paged_attention(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
     ``tile_keys_total``, ``tile_keys_max``); everything else, and float32 always, takes the general
     kernel.  Every choice computes the same function.  ``bias`` (float32 [nq, rows]) is a bias by distance on the
     scores (``bias_log2``: the same times log2(e), which the matrix-core kernels add to their exponents of two);
-    ``gate`` [T, >= nq]: every head's output is multiplied by the sigmoid of its gate."""
+    ``gate`` [T, >= nq]: every head's output is multiplied by the sigmoid of its gate; ``sink`` (float32 [nq]):
+    exp(sink[head]) joins the softmax's denominator (``sink_log2``: the same times log2(e))."""
     if not attention_mfma_supports(q.dtype, hd, group.page_size, nq, nkv):
         if q.dtype == torch.bfloat16:
             _warn_general_attention(hd, group.page_size)
         out = paged_attention_generic(q, k_pool, v_pool, ctx.positions, ctx.token_entry, group.block_table,
-                                      group.page_size, nq, nkv, hd, scale, window, bias=bias)
+                                      group.page_size, nq, nkv, hd, scale, window, bias=bias, sink=sink)
         return out if gate is None else head_gate_(out, gate, nq, hd)
     if bias is not None:
         _need(bias_log2 is not None and bias_log2.shape == bias.shape, "the matrix-core kernels take the bias times log2(e)")
+    if sink is not None:
+        _need(sink_log2 is not None and sink_log2.shape == sink.shape, "the matrix-core kernels take the sinks times log2(e)")
     _need(plan is not None, "the matrix-core attention kernels need the step's work lists (a step plan)")
     out = torch.empty((q.shape[0], nq * hd), dtype=q.dtype, device=q.device)
     n = plan.facts
     if n["num_decode"]:
         attention_decode_mfma(q, out, k_pool, v_pool, plan.arrays["decode_tokens"], n["num_decode"], ctx.positions,
                               ctx.token_entry, group.block_table, group.page_size, nq, nkv, hd, scale, window,
-                              n["max_decode_kv"], bias_log2=bias_log2 if bias is not None else None, gate=gate)
+                              n["max_decode_kv"], bias_log2=bias_log2 if bias is not None else None, gate=gate,
+                              sink_log2=sink_log2 if sink is not None else None)
     if n["num_tiles"]:
         attention_prefill_mfma(q, out, k_pool, v_pool, plan.arrays["tiles"], n["num_tiles"], ctx.positions,
                                ctx.token_entry, group.block_table, group.page_size, nq, nkv, hd, scale, window,
                                keys_total=n["tile_keys_total"], keys_max=n["tile_keys_max"],
-                               bias_log2=bias_log2 if bias is not None else None, gate=gate)
+                               bias_log2=bias_log2 if bias is not None else None, gate=gate,
+                               sink_log2=sink_log2 if sink is not None else None)
+    return out
+
+
+# ---------------------------------------------------------------------------------- routed feed-forward
+
+MOE_MAX_ROUTER, MOE_MAX_TOP = 1024, 32
+MOE_TILE_ROWS = (16, 32, 64)     # grouped rows a block of the matrix-core expert products takes
+
+
+def moe_route(logits: torch.Tensor, correction: Optional[torch.Tensor], top: int):
+    """(ids int32 [T, top], weights float32 [T, top]) from router logits float32 [T, R]: the softmax over all R, the
+    ``top`` largest of softmax + ``correction`` (float32 [R] or None; ties go to the lower index), and as weights the
+    chosen outputs' softmax values over their sum (+ 1e-20)."""
+    T, R = logits.shape
+    _need(logits.dtype == torch.float32 and logits.stride(1) == 1, "router logits must be float32 [T, R]")
+    _need(1 <= top <= min(R, MOE_MAX_TOP) and R <= MOE_MAX_ROUTER, f"top {top} of {R} router outputs: at most "
+          f"{MOE_MAX_TOP} of {MOE_MAX_ROUTER}")
+    if correction is not None:
+        _need(correction.dtype == torch.float32 and correction.numel() == R and correction.is_contiguous(),
+              "the router's correction must be float32 [R]")
+    ids = torch.empty((T, top), dtype=torch.int32, device=logits.device)
+    weights = torch.empty((T, top), dtype=torch.float32, device=logits.device)
+    _check(build.load("moe").ullm_moe_route(_p(logits), _c_int(logits.stride(0)), _p(correction), _c_int(T), _c_int(R),
+                                            _c_int(top), _p(ids), _p(weights), _stream()), "moe_route")
+    return ids, weights
+
+
+def moe_max_tiles(n_pairs: int, n_experts: int, tile_rows: int) -> int:
+    """The most tiles of ``tile_rows`` rows that ``n_pairs`` (token, expert) pairs over ``n_experts`` experts can fill."""
+    return max(1, n_pairs // tile_rows + min(n_experts, n_pairs))
+
+
+def moe_sort(ids: torch.Tensor, n_experts: int, tile_rows: int):
+    """Groups the pairs (token, k) of ``ids`` int32 [T, top] by expert.  Returns (slot_of_pair int32 [T * top], -1 for
+    a pair whose expert index is >= ``n_experts``; token_of_slot int32 [T * top]; tiles int32 [max_tiles, 3] =
+    (expert, first slot, rows <= tile_rows), rows 0 in unused tiles; offsets int32 [n_experts + 1])."""
+    _i32(ids, "ids")
+    T, top = ids.shape
+    n_pairs = T * top
+    dev = ids.device
+    max_tiles = moe_max_tiles(n_pairs, n_experts, tile_rows)
+    slot_of_pair = torch.empty(n_pairs, dtype=torch.int32, device=dev)
+    token_of_slot = torch.empty(n_pairs, dtype=torch.int32, device=dev)
+    tiles = torch.empty((max_tiles, 3), dtype=torch.int32, device=dev)
+    offsets = torch.empty(n_experts + 1, dtype=torch.int32, device=dev)
+    _check(build.load("moe").ullm_moe_sort(_p(ids), _c_int(n_pairs), _c_int(top), _c_int(n_experts), _c_int(tile_rows),
+                                           _p(offsets), _p(slot_of_pair), _p(token_of_slot), _p(tiles), _c_int(max_tiles),
+                                           _stream()), "moe_sort")
+    return slot_of_pair, token_of_slot, tiles, offsets
+
+
+def moe_rows(x: torch.Tensor, row_index: Optional[torch.Tensor], w: torch.Tensor, tiles: torch.Tensor, tile_rows: int,
+             n_slots: int, gated: bool, limit: float = 0.0, alpha: float = 0.0) -> torch.Tensor:
+    """The experts' products over grouped rows.  ``w`` is [experts, 2 n_out, K] (``gated``: gate rows, then up rows) or
+    [experts, n_out, K]; row ``slot`` of the result comes from row ``row_index[slot]`` of ``x`` (``slot`` itself
+    without an index) and the expert of the tile that holds the slot.  Gated: the clamped gated unit of the two
+    products in x's dtype [n_slots, n_out]; else the product in float32.  Rows of slots no tile holds stay
+    unwritten."""
+    _need(w.dim() == 3 and w.is_contiguous() and w.dtype == x.dtype, "expert matrices must be contiguous [experts, rows, K] of x's dtype")
+    K = w.shape[2]
+    n_out = w.shape[1] // 2 if gated else w.shape[1]
+    _need(x.dim() == 2 and x.shape[1] == K and x.stride(1) == 1, "x must be [rows, K]")
+    _need(not gated or w.shape[1] % 2 == 0, "gated expert matrices hold gate rows, then as many up rows")
+    _need(tiles.dtype == torch.int32 and tiles.dim() == 2 and tiles.shape[1] == 3 and tiles.is_contiguous(), "tiles must be int32 [n, 3]")
+    if row_index is not None:
+        _i32(row_index, "row_index", n_slots)
+    else:
+        _need(x.shape[0] >= n_slots, "fewer rows than slots")
+    out = torch.empty((n_slots, n_out), dtype=x.dtype if gated else torch.float32, device=x.device)
+    _check(build.load("moe").ullm_moe_rows(_p(x), _c_int(x.stride(0)), _p(row_index), _p(w), _p(tiles),
+                                           _c_int(tiles.shape[0]), _c_int(tile_rows), _p(out), _c_int(out.stride(0)),
+                                           _c_int(n_out), _c_int(K), _c_int(1 if gated else 0), _c_float(limit),
+                                           _c_float(alpha), _c_int(_dt(x)), _stream()), "moe_rows")
+    return out
+
+
+def moe_combine(y: Optional[torch.Tensor], x: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor,
+                slot_of_pair: torch.Tensor, n_experts: int, base: Optional[torch.Tensor] = None,
+                bias: Optional[torch.Tensor] = None, shared: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """float32 [T, H]: ``base`` + ``bias`` + ``shared`` + the sum over a token's chosen experts, in their order, of
+    weight times the expert's row of ``y`` (float32 [slots, H]) or, for an expert index >= ``n_experts``, times the
+    token's own row of ``x``."""
+    T, H = x.shape
+    top = ids.shape[1]
+    _need(x.stride(1) == 1, "x must have unit stride along its rows")
+    _need(y is None or (y.dtype == torch.float32 and y.dim() == 2 and y.shape[1] == H and y.is_contiguous()), "y must be float32 [slots, H]")
+    _need(y is not None or n_experts == 0, "experts with weights need their rows")
+    _i32(ids, "ids", T * top)
+    _i32(slot_of_pair, "slot_of_pair", T * top)
+    _need(weights.dtype == torch.float32 and weights.is_contiguous() and weights.numel() == T * top, "weights must be float32 [T, top]")
+    base_dt = F32
+    if base is not None:
+        _need(base.shape == (T, H) and base.is_contiguous(), "base must be contiguous [T, H]")
+        base_dt = _dt(base)
+    if bias is not None:
+        _need(bias.dtype == torch.float32 and bias.numel() == H and bias.is_contiguous(), "bias must be float32 [H]")
+    if shared is not None:
+        _need(shared.shape == (T, H) and shared.is_contiguous() and shared.dtype == x.dtype, "shared must be [T, H] of x's dtype")
+    out = torch.empty((T, H), dtype=torch.float32, device=x.device)
+    _check(build.load("moe").ullm_moe_combine(_p(y), _p(x), _c_int(x.stride(0)), _p(ids), _p(weights), _p(slot_of_pair),
+                                              _c_int(top), _c_int(n_experts), _p(base), _c_int(base_dt), _p(bias),
+                                              _p(shared), _p(out), _c_int(T), _c_int(H), _c_int(_dt(x)), _stream()),
+           "moe_combine")
     return out
 
 

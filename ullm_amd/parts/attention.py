@@ -11,11 +11,16 @@ query/key size (``value_dim``), the q/k norm taken over the whole projection ins
 (``qk_norm="whole"``, gains of the projections' full sizes), a bias on the scores by distance (a position part
 with ``score_bias()``), a gate per head on the heads' outputs (``head_gate``: sigmoid of one more projection of
 the mixer's input), no key/value projections of its own (``own_kv=False``: the layer reads the cache another
-layer writes), and other tensor names (``names``).  Any of these takes the general path below: one projection
+layer writes), values that are the keys as projected, before rotation (``values="keys"``: no value projection),
+a sink per head in the softmax's denominator (``sink``: a learned number with no key and no value), biases on the
+projections also there (``bias`` on q, k and v, ``out_bias`` on the output) and other tensor names (``names``).
+Any of these takes the general path below: one projection
 q | k | v | gate, heads padded with zeros to a size the attention kernels take (zero key dims add nothing to a
 score, zero value dims give zero outputs that meet zero columns of the output projection).
 """
 from __future__ import annotations
+
+import math
 
 from typing import Dict, List, Optional
 
@@ -34,7 +39,9 @@ from .linear import add_into_stream, can_fuse, linear, linear_into_stream, linea
 FUSED_DECODE_MAX_TOKENS = 64
 
 DEFAULT_NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
-                 "q_norm": "q_norm.weight", "k_norm": "k_norm.weight", "gate": "gate_proj.weight"}
+                 "q_norm": "q_norm.weight", "k_norm": "k_norm.weight", "gate": "gate_proj.weight",
+                 "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias", "o_bias": "o_proj.bias",
+                 "sink": "sinks"}
 KERNEL_HEAD_SIZES = (32, 64, 96, 128, 256)      # what the matrix-core attention kernels take
 
 
@@ -85,18 +92,23 @@ class GQAttention(Mixer):
                  position: Optional[PositionEncoding] = None, qk_norm_eps: Optional[float] = None,
                  bias: bool = False, window: int = 0, scale: Optional[float] = None,
                  value_dim: Optional[int] = None, qk_norm: str = "head", head_gate: bool = False,
-                 own_kv: bool = True, names: Optional[Dict[str, str]] = None):
+                 own_kv: bool = True, names: Optional[Dict[str, str]] = None, values: str = "own",
+                 sink: bool = False, out_bias: bool = False):
         if qk_norm not in ("head", "whole"):
             raise ValueError(f"qk_norm={qk_norm!r}: 'head' (per head) or 'whole' (over the whole projection)")
+        if values not in ("own", "keys"):
+            raise ValueError(f"values={values!r}: 'own' (a value projection) or 'keys' (the keys as projected)")
         self.dim, self.vdim = head_dim, head_dim if value_dim is None else int(value_dim)
         self.qk_norm, self.head_gate, self.own_kv = qk_norm, bool(head_gate), bool(own_kv)
+        self.values_are_keys, self.sink, self.out_bias = values == "keys", bool(sink), bool(out_bias)
         self.names = {**DEFAULT_NAMES, **(names or {})}
         self.general = (self.vdim != head_dim or qk_norm == "whole" or self.head_gate or not self.own_kv
-                        or names is not None or (position is not None and type(position).score_bias
-                                                 is not PositionEncoding.score_bias))
+                        or names is not None or self.values_are_keys or self.sink or self.out_bias
+                        or (position is not None and type(position).score_bias is not PositionEncoding.score_bias))
         if self.general:
-            if bias:
-                raise ValueError("projection biases are not built for the general attention path")
+            if self.values_are_keys and (self.vdim != head_dim or qk_norm == "whole" or not self.own_kv):
+                raise ValueError("values that are the keys need keys of the layer's own, of the values' size, "
+                                 "and no norm over the whole projection")
             padded = padded_head_size(head_dim, self.vdim)
             if qk_norm == "head" and qk_norm_eps is not None and padded != head_dim:
                 raise ValueError(f"a per-head norm over heads of {head_dim} stored as {padded}: not built")
@@ -112,7 +124,8 @@ class GQAttention(Mixer):
         self.bias = bias
         self.window = int(window)
         self.scale = float(scale) if scale is not None else self.dim ** -0.5   # qwen3.py:81
-        self.w_qkv = self.b_qkv = self.w_o = self.q_gain = self.k_gain = None
+        self.w_qkv = self.b_qkv = self.w_o = self.b_o = self.q_gain = self.k_gain = None
+        self.sinks = self.sinks_log2 = None
 
     def children(self):
         return [self.position] if self.position is not None else []
@@ -201,7 +214,19 @@ class GQAttention(Mixer):
         H, nq, nkv, d, dv = self.hidden_size, self.nq, self.nkv, self.dim, self.vdim
         out = [WeightDecl(self._name("q"), (nq * d, H)), WeightDecl(self._name("o"), (H, nq * dv))]
         if self.own_kv:
-            out += [WeightDecl(self._name("k"), (nkv * d, H)), WeightDecl(self._name("v"), (nkv * dv, H))]
+            out.append(WeightDecl(self._name("k"), (nkv * d, H)))
+            if not self.values_are_keys:
+                out.append(WeightDecl(self._name("v"), (nkv * dv, H)))
+        if self.bias:
+            out.append(WeightDecl(self._name("q_bias"), (nq * d,), keep_fp32=True))
+            if self.own_kv:
+                out.append(WeightDecl(self._name("k_bias"), (nkv * d,), keep_fp32=True))
+                if not self.values_are_keys:
+                    out.append(WeightDecl(self._name("v_bias"), (nkv * dv,), keep_fp32=True))
+        if self.out_bias:
+            out.append(WeightDecl(self._name("o_bias"), (H,), keep_fp32=True))
+        if self.sink:
+            out.append(WeightDecl(self._name("sink"), (nq,), keep_fp32=True))
         if self.qk_norm_eps is not None:
             per = d if self.qk_norm == "head" else None
             out.append(WeightDecl(self._name("q_norm"), (per or nq * d,), init="gain", keep_fp32=True))
@@ -225,14 +250,28 @@ class GQAttention(Mixer):
             return out.view((heads * hd,) + tuple(t.shape[1:]))
 
         pieces = [heads_padded(tensors[self._name("q")], nq, d)]
+        biases = [heads_padded(tensors[self._name("q_bias")], nq, d)] if self.bias else []
         self.q_off, self.k_off, self.v_off = 0, nq * hd, (nq + nkv) * hd
         if self.own_kv:
-            pieces += [heads_padded(tensors[self._name("k")], nkv, d), heads_padded(tensors[self._name("v")], nkv, dv)]
+            pieces.append(heads_padded(tensors[self._name("k")], nkv, d))
+            if self.bias:
+                biases.append(heads_padded(tensors[self._name("k_bias")], nkv, d))
+            if not self.values_are_keys:
+                pieces.append(heads_padded(tensors[self._name("v")], nkv, dv))
+                if self.bias:
+                    biases.append(heads_padded(tensors[self._name("v_bias")], nkv, dv))
         self.gate_off = sum(p.shape[0] for p in pieces)
         if self.head_gate:
             gate = tensors[self._name("gate")]
             pieces.append(torch.cat((gate, gate.new_zeros((-nq % 8, H))), dim=0))
+            if self.bias:
+                biases.append(biases[0].new_zeros((pieces[-1].shape[0],)))
         self.w_qkv = torch.cat(pieces, dim=0).contiguous()
+        self.b_qkv = torch.cat(biases, dim=0).contiguous() if self.bias else None
+        self.b_o = tensors[self._name("o_bias")].contiguous() if self.out_bias else None
+        if self.sink:
+            self.sinks = tensors[self._name("sink")].to(torch.float32).contiguous()
+            self.sinks_log2 = (self.sinks * math.log2(math.e)).contiguous()
         w_o = tensors[self._name("o")]
         if dv != hd:
             wide = w_o.new_zeros((H, nq, hd))
@@ -254,13 +293,15 @@ class GQAttention(Mixer):
         nq, nkv, hd = self.nq, self.nkv, self.hd
         T = x.shape[0]
         group = ctx.groups[cache.group]
-        proj = linear(x, self.w_qkv)
+        proj = linear(x, self.w_qkv, self.b_qkv)
         q = torch.empty((T, nq * hd), dtype=proj.dtype, device=proj.device)
         table, rot, style = self.position.kernel_args() if self.position is not None else (None, 0, 0)
         if self.qk_norm == "head" and self.own_kv:
-            ops.qk_norm_rope_write(proj[:, :(nq + 2 * nkv) * hd], q, self.q_gain, self.k_gain, self.qk_norm_eps or 0.0,
+            kv_heads = nkv if self.values_are_keys else 2 * nkv
+            ops.qk_norm_rope_write(proj[:, :(nq + kv_heads) * hd], q, self.q_gain, self.k_gain, self.qk_norm_eps or 0.0,
                                    table, rot, style, ctx.positions, ctx.token_entry, group.block_table, cache.k_pool,
-                                   cache.v_pool, group.page_size, nq, nkv, hd, write_kv=True)
+                                   cache.v_pool, group.page_size, nq, nkv, hd, write_kv=True,
+                                   values_from_keys=self.values_are_keys)
         else:
             if style != 0 and rot > 0 or (self.qk_norm == "head" and self.qk_norm_eps is not None):
                 raise NotImplementedError("rotation or a per-head norm without keys of the layer's own: not built")
@@ -273,5 +314,9 @@ class GQAttention(Mixer):
         out = ops.paged_attention(q, cache.k_pool, cache.v_pool, ctx, group, nq, nkv, hd, self.scale, self.window,
                                   ctx.plans["attention"], bias=bias,
                                   bias_log2=self.position.score_bias_log2() if bias is not None else None,
-                                  gate=proj[:, self.gate_off:] if self.head_gate else None)
+                                  gate=proj[:, self.gate_off:] if self.head_gate else None,
+                                  sink=self.sinks, sink_log2=self.sinks_log2)
+        if self.b_o is not None:
+            # the bias joins the 32-bit sums of the product, which stay 32-bit on their way to the stream
+            return linear(out, self.w_o, self.b_o, out_dtype=torch.float32)
         return linear_into_stream(out, self.w_o, ctx)

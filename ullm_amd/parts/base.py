@@ -312,9 +312,10 @@ class NormedBranch:
     """A branch output that joins the stream as ``mult * norm(branch) * gain``: the norm behind a mixer or
     feed-forward of a block that norms on both sides of each.  It is handed on as the pending branch, and the
     norm that adds it (``Norm.add_norm``) applies ``post`` (a :class:`Norm` with ``kernel_form()``), the
-    multiplier, the add and its own norm in one pass over the row."""
-    branch: torch.Tensor          # [T, hidden] in the compute dtype
-    post: "Norm"
+    multiplier, the add and its own norm in one pass over the row.  Without ``post`` the branch joins the
+    stream as ``mult * branch`` (a block that only scales what it adds)."""
+    branch: torch.Tensor          # [T, hidden] in the compute dtype or float32
+    post: Optional["Norm"]
     mult: float = 1.0
 
 

@@ -9,6 +9,9 @@ from __future__ import annotations
 
 from typing import Optional
 
+import torch
+
+from ..kernels import ops
 from .base import Block, FeedForward, LayerCache, Mixer, Norm, NormedBranch, PendingNorm, StepContext, register_part
 
 
@@ -107,3 +110,38 @@ class SandwichBlock(Block):
 def _one_branch(y):
     """A stack of partial sums [S, T, hidden] added up: a norm behind the branch needs the whole rows."""
     return y.sum(0).contiguous() if y.dim() == 3 else y
+
+
+@register_part("block", "parallel")
+class ParallelBlock(Block):
+    """One norm whose output both sublayers read, and a multiplier on their sum:
+    h = norm(x); x += mult * (mixer(h) + ffn(h)).  A block without a feed-forward (``ffn`` None) adds the mixer
+    alone.  The sum of the two branches is 32-bit and travels on as the pending branch; the next norm of the
+    stream multiplies, adds and norms in one pass.  A feed-forward that offers ``forward_onto(x, ctx, base)`` adds
+    its result onto the mixer's in its own last kernel."""
+
+    def __init__(self, norm: Norm, mixer: Mixer, ffn: Optional[FeedForward] = None, mult: float = 1.0):
+        self.norm, self.mixer, self.ffn, self.mult = norm, mixer, ffn, float(mult)
+
+    def children(self):
+        return [p for p in (self.norm, self.mixer, self.ffn) if p is not None]
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    def entry_norm(self):
+        return self.norm
+
+    def forward(self, residual, pending, ctx: StepContext, cache: LayerCache):
+        if isinstance(pending, PendingNorm):
+            pending = None                               # the stream is complete; this block norms it itself
+        h = self.norm.add_norm(pending, residual, out_dtype=ctx.dtype)
+        mixed = _one_branch(self.mixer.forward(h, ctx, cache))
+        if self.ffn is None:
+            return residual, NormedBranch(mixed, None, self.mult)
+        if hasattr(self.ffn, "forward_onto"):
+            return residual, NormedBranch(self.ffn.forward_onto(h, ctx, mixed), None, self.mult)
+        total = torch.zeros(mixed.shape, dtype=torch.float32, device=mixed.device)
+        ops.residual_add(mixed, total)
+        ops.residual_add(_one_branch(self.ffn.forward(h, ctx)), total)
+        return residual, NormedBranch(total, None, self.mult)

@@ -49,11 +49,14 @@ class RMSNorm(Norm):
 
 def add_normed_branch(branch: NormedBranch, residual, form, rows, out_dtype):
     """The stream takes ``mult * post(branch)`` and is normed by ``form`` = (gain, eps, kind), in one kernel."""
-    post = branch.post.kernel_form()
-    if post is None:
-        raise TypeError(f"{type(branch.post).__name__} cannot stand behind a branch: it has no kernel form")
     gain, eps, kind = form
-    post_gain, post_eps, post_kind = post
+    if branch.post is None:                    # the branch joins the stream times the multiplier, unnormed
+        post_gain, post_eps, post_kind = None, 0.0, ops.NORM_RMS
+    else:
+        post = branch.post.kernel_form()
+        if post is None:
+            raise TypeError(f"{type(branch.post).__name__} cannot stand behind a branch: it has no kernel form")
+        post_gain, post_eps, post_kind = post
     return ops.add_norm_general(branch.branch, residual, gain, eps, kind, out_dtype or branch.branch.dtype, rows=rows,
                                 post_gain=post_gain, post_eps=post_eps, post_kind=post_kind, mult=branch.mult)
 
