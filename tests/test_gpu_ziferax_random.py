@@ -1,0 +1,125 @@
+"""Ziferax configurations drawn at random (sizes, heads, windows, rotated dims, experts, identity experts, top counts,
+shared experts, layers that use another's tensors, layers without a feed-forward) through the replayer: in 32-bit
+against the plain 64-bit implementation, whole prompts, portions of drawn sizes followed by single tokens, and a
+schedule of up to four live requests in a pool and slots that are used again; in bfloat16 the same schedules
+against the engine's own whole prompts (what rounding does to a routed model is bounded in the tests of the fixed
+models; here only the cutting must not matter)."""
+import json
+import os
+import random
+
+import numpy as np
+import pytest
+from safetensors.torch import save_file
+
+import plain_ziferax as plain
+from gpu_util import DEV
+
+pytestmark = pytest.mark.gpu
+
+
+def drawn_layer(rng):
+    kv = rng.choice([1, 1, 2, 3, 4])
+    dim = rng.choice([8, 16, 24, 32, 40, 48, 64, 80, 96, 128])
+    rot = rng.choice([0, 2, dim // 2 - (dim // 2) % 2, dim])
+    mixer = dict(heads=kv * rng.choice([1, 2, 3, 4, 8]), kv_heads=kv, dim=dim, vdim=dim,
+                 mask=dict(size=rng.choice([1, 2, 5, 15, 16, 17, 31, 32, 33, 48, 64, 100, 500])),
+                 rot=dict(base=rng.choice([100.0, 10000.0, 500000.0]), dims=rot), scale=rng.choice([0.05, 0.125, 0.3]))
+    if rot == 0:
+        del mixer["rot"]
+    mlp = None
+    if rng.random() < 0.8:
+        experts, identity = rng.choice([1, 2, 3, 5, 8, 16, 40]), rng.choice([0, 0, 1, 2, 5])
+        mlp = dict(kind="moe", router=dict(experts=experts, identity=identity, top=rng.randint(1, min(6, experts + identity))),
+                   expert=dict(ff=rng.choice([4, 8, 12, 16, 24, 40, 64, 100]), limit=rng.choice([0.5, 1.5, 7.0])))
+        if rng.random() < 0.6:
+            mlp["shared"] = dict(ff=rng.choice([8, 20, 64, 136]), limit=rng.choice([0.5, 2.0]))
+    return dict(type="attention", mixer=mixer, mlp=mlp)
+
+
+def drawn_config(rng):
+    layers = []
+    for i in range(rng.randint(1, 5)):
+        own = [j for j, L in enumerate(layers) if "weights_of" not in L]
+        if own and rng.random() < 0.3:
+            src = rng.choice(own)
+            layers.append(dict(json.loads(json.dumps(layers[src])), weights_of=src))
+        else:
+            layers.append(drawn_layer(rng))
+    return dict(architecture="Ziferax", vocab=rng.randint(40, 700), width=rng.choice([24, 32, 40, 48, 64, 72, 96, 128, 160, 256]),
+                layers=layers, norm=dict(eps=rng.choice([1e-5, 1e-6, 1e-3])), residual_mult=rng.choice([0.3, 0.5, 1.0, 0.7]))
+
+
+def worst_error(got, want):
+    return float(np.abs(got - want).max() / np.abs(want).max())
+
+
+def schedules(rep, rng, reqs):
+    """{request: logits of every position} for r0 whole ("whole"), r0 in drawn portions ("cut"), and all requests in a
+    drawn schedule of up to four live ones ("mixed": {request: logits})."""
+    toks = reqs["r0"]
+    whole = rep.step({"step": 0, "entries": [{"id": "w", "tokens": toks, "want": list(range(len(toks)))}], "end": ["w"]})
+    at, step, parts = 0, 0, []
+    sizes = [rng.choice([2, 3, 5, 16, 17, 31]) for _ in range(4)] + [1] * len(toks)
+    while at < len(toks):
+        n = min(sizes[step], len(toks) - at)
+        parts.append(rep.step({"step": step, "entries": [{"id": "c", "tokens": toks[at:at + n], "want": list(range(n))}],
+                               "end": ["c"] if at + n == len(toks) else []}))
+        at, step = at + n, step + 1
+    waiting, live, at, got = list(reqs), [], {}, {k: [] for k in reqs}
+    step = 0
+    while waiting or live:
+        while waiting and len(live) < 4 and rng.random() < 0.7:
+            k = waiting.pop(0)
+            live.append(k)
+            at[k] = 0
+        entries, end = [], []
+        for k in list(live):
+            if rng.random() < 0.25 and len(live) > 1:
+                continue
+            n = min(len(reqs[k]) - at[k], rng.choice([1, 1, 1, 2, 3, 7, 16, 17, 40]))
+            entries.append({"id": k, "tokens": reqs[k][at[k]:at[k] + n], "want": list(range(n))})
+            at[k] += n
+            if at[k] == len(reqs[k]):
+                end.append(k)
+                live.remove(k)
+        if not entries:
+            continue
+        out, o = rep.step({"step": step, "entries": entries, "end": end}), 0
+        for e in entries:
+            got[e["id"]].append(out[o:o + len(e["tokens"])])
+            o += len(e["tokens"])
+        step += 1
+    return whole, np.concatenate(parts), {k: np.concatenate(v) for k, v in got.items()}
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_drawn_configurations(seed, tmp_path):
+    from ullm_amd.replay import Replayer
+    rng = random.Random(7000 + seed)
+    cfg = drawn_config(rng)
+    w = plain.random_weights(cfg, seed)
+    with open(os.path.join(tmp_path, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    save_file({k: v.contiguous() for k, v in w.items()}, os.path.join(tmp_path, "model.safetensors"))
+    wide = {k: v.double() for k, v in w.items()}
+    reqs = {f"r{i}": [rng.randrange(cfg["vocab"]) for _ in range(rng.randint(20, 110))] for i in range(6)}
+    want = {k: plain.forward(wide, cfg, t).float().numpy() for k, t in reqs.items()}
+    state = rng.getstate()
+    whole, cut, mixed = schedules(Replayer(str(tmp_path), "float32", 512, 16, DEV, max_requests=4), rng, reqs)
+    assert worst_error(whole, want["r0"]) <= 3e-5 and worst_error(cut, want["r0"]) <= 3e-5
+    for k in reqs:
+        assert worst_error(mixed[k], want[k]) <= 3e-5, k
+    # bfloat16: the same schedules; a position's logits do not depend on the cutting beyond rounding (a row count picks
+    # the product kernel, so sums may be ordered otherwise, and a close call of a router may then fall otherwise: most
+    # rows agree to rounding, every row far inside what a lost key or a stale slot would do)
+    rng.setstate(state)
+    rep = Replayer(str(tmp_path), "bfloat16", 512, 16, DEV, max_requests=4)
+    whole, cut, mixed = schedules(rep, rng, reqs)
+    alone = {k: rep.step({"step": 0, "entries": [{"id": "a", "tokens": t, "want": list(range(len(t)))}], "end": ["a"]})
+             for k, t in reqs.items()}
+    for got, ref in [(cut, whole)] + [(mixed[k], alone[k]) for k in reqs]:
+        err = np.abs(got - ref).max(-1) / np.abs(ref).max()
+        assert np.median(err) <= 1.5e-2 and err.max() <= 0.3, (float(np.median(err)), float(err.max()))
+    err = np.abs(whole - want["r0"]).max(-1) / np.abs(want["r0"]).max()
+    assert np.median(err) <= 4e-2 and err.max() <= 0.5, (float(np.median(err)), float(err.max()))
