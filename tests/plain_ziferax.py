@@ -102,20 +102,25 @@ def experts(w, prefix: str, mlp: dict, h: torch.Tensor) -> torch.Tensor:
     return out
 
 
-def forward(w, cfg: dict, tokens: List[int], streams: Optional[list] = None) -> torch.Tensor:
-    """Logits [len(tokens), vocab]; with ``streams`` the residual stream after every layer is appended to it."""
+def forward(w, cfg: dict, tokens: List[int], streams: Optional[list] = None, round_to=None) -> torch.Tensor:
+    """Logits [len(tokens), vocab]; with ``streams`` the residual stream after every layer is appended to it.
+    With ``round_to`` (a dtype) every normed layer input and the head's input is rounded to it and widened again:
+    what rounding of the sublayers' inputs alone does to the logits, a floor for any engine that computes in it."""
+    def rounded(h):
+        return h if round_to is None else h.to(round_to).to(h.dtype)
+
     x = w["embed"][torch.tensor(tokens)]
     eps, mult = cfg["norm"]["eps"], cfg.get("residual_mult", 1.0)
     for i, L in enumerate(cfg["layers"]):
         p = f"l{L['weights_of'] if L.get('weights_of') is not None else i}"
-        h = rms(x, eps) * w[f"{p}.norm1"]
+        h = rounded(rms(x, eps) * w[f"{p}.norm1"])
         y = attention(w, f"{p}.mix", L["mixer"], h)
         if L.get("mlp") is not None:
             y = y + experts(w, f"{p}.mlp", L["mlp"], h)
         x = x + mult * y
         if streams is not None:
             streams.append(x.clone())
-    return (rms(x, eps) * w["final.norm"]) @ w["embed"].T
+    return rounded(rms(x, eps) * w["final.norm"]) @ w["embed"].T
 
 
 def greedy_generate(w, cfg, prompt: List[int], n: int) -> List[int]:

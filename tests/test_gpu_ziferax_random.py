@@ -10,6 +10,7 @@ import random
 
 import numpy as np
 import pytest
+import torch
 from safetensors.torch import save_file
 
 import plain_ziferax as plain
@@ -105,21 +106,27 @@ def test_drawn_configurations(seed, tmp_path):
     wide = {k: v.double() for k, v in w.items()}
     reqs = {f"r{i}": [rng.randrange(cfg["vocab"]) for _ in range(rng.randint(20, 110))] for i in range(6)}
     want = {k: plain.forward(wide, cfg, t).float().numpy() for k, t in reqs.items()}
+    narrow = {k: v.float() for k, v in w.items()}
+    # what 32-bit sums alone do to this model (four times that, as the engine sums in another order), at least 3e-5
+    bound = {k: max(3e-5, 4 * worst_error(plain.forward(narrow, cfg, t).numpy(), want[k])) for k, t in reqs.items()}
     state = rng.getstate()
     whole, cut, mixed = schedules(Replayer(str(tmp_path), "float32", 512, 16, DEV, max_requests=4), rng, reqs)
-    assert worst_error(whole, want["r0"]) <= 3e-5 and worst_error(cut, want["r0"]) <= 3e-5
+    assert worst_error(whole, want["r0"]) <= bound["r0"] and worst_error(cut, want["r0"]) <= bound["r0"]
+    assert np.array_equal(whole, cut)                       # 32-bit sums are ordered by the row alone
     for k in reqs:
-        assert worst_error(mixed[k], want[k]) <= 3e-5, k
-    # bfloat16: the same schedules; a position's logits do not depend on the cutting beyond rounding (a row count picks
-    # the product kernel, so sums may be ordered otherwise, and a close call of a router may then fall otherwise: most
-    # rows agree to rounding, every row far inside what a lost key or a stale slot would do)
+        assert worst_error(mixed[k], want[k]) <= bound[k], k
+    # bfloat16: the same schedules.  What rounding does to a routed model depends on the model (a rounded router input
+    # picks another expert at a close call, and then a whole row moves), so the bounds are multiples of what the plain
+    # implementation loses when nothing but its sublayers' inputs are rounded to bfloat16: for the middle row and for
+    # 85 rows of 100; single rows may move further.  A position's logits do not depend on the cutting beyond that.
     rng.setstate(state)
     rep = Replayer(str(tmp_path), "bfloat16", 512, 16, DEV, max_requests=4)
     whole, cut, mixed = schedules(rep, rng, reqs)
     alone = {k: rep.step({"step": 0, "entries": [{"id": "a", "tokens": t, "want": list(range(len(t)))}], "end": ["a"]})
              for k, t in reqs.items()}
-    for got, ref in [(cut, whole)] + [(mixed[k], alone[k]) for k in reqs]:
+    floor = np.concatenate([np.abs(plain.forward(wide, cfg, t, round_to=torch.bfloat16).float().numpy() - want[k]).max(-1)
+                            / np.abs(want[k]).max() for k, t in reqs.items()])
+    mid, most = 5e-3 + 4 * float(np.median(floor)), 1e-2 + 4 * float(np.quantile(floor, 0.85))
+    for got, ref in [(whole, want["r0"]), (cut, whole)] + [(mixed[k], alone[k]) for k in reqs]:
         err = np.abs(got - ref).max(-1) / np.abs(ref).max()
-        assert np.median(err) <= 1.5e-2 and err.max() <= 0.3, (float(np.median(err)), float(err.max()))
-    err = np.abs(whole - want["r0"]).max(-1) / np.abs(want["r0"]).max()
-    assert np.median(err) <= 4e-2 and err.max() <= 0.5, (float(np.median(err)), float(err.max()))
+        assert np.median(err) <= mid and np.quantile(err, 0.85) <= most, (float(np.median(err)), float(np.quantile(err, 0.85)), mid, most)
