@@ -55,8 +55,9 @@ def parse_args():
                     help="instead of the default workload: Pamopel (attention with a distance bias and head gates, a "
                          "layer on another's keys and values, a Mamba-2 layer) beside a Qwen3 stack of the same width, "
                          f"heads, feed-forward, vocabulary and depth, random weights; shapes: {sorted(DESIGN_SHAPES)}")
-    ap.add_argument("--design-model", choices=("both", "pamopel", "qwen3"), default="both",
-                    help="with --design: run one of the two designs only (for profiles)")
+    ap.add_argument("--design-model", choices=("both", "all", "pamopel", "qwen3", "ziferax"), default="both",
+                    help="with --design: one design only (for profiles), Pamopel and Qwen3 (both), or these and Ziferax "
+                         "(all: a stack of parallel blocks of windowed attention with sinks and a routed feed-forward)")
     ap.add_argument("--prefill-only", type=int, default=0, metavar="T",
                     help="only time a T-token prompt and print its figures (for profiling)")
     return ap.parse_args()
@@ -154,12 +155,24 @@ def design_configs(shape):
     return pamopel, qwen
 
 
+# Ziferax at a design shape: the same width, heads and depth; a window of 1024 keys, half of each head rotated; per
+# token as many feed-forward columns as the dense stack has (top 4 of 32 experts of a sixth of it each, four identity
+# experts beside them, and a shared expert of a third of it), so a token's products are of equal size.
+def ziferax_config(shape):
+    (W, H, G, D, F, L), _ = DESIGN_SHAPES[shape]
+    mixer = dict(heads=H, kv_heads=G, dim=D, vdim=D, scale=D ** -0.5, mask=dict(size=1024), rot=dict(base=500000.0, dims=D // 2))
+    mlp = dict(kind="moe", router=dict(experts=32, identity=4, top=4), expert=dict(ff=F // 6, limit=7.0),
+               shared=dict(ff=F // 3, limit=7.0))
+    return dict(architecture="Ziferax", vocab=DESIGN_VOCAB, width=W, norm=dict(eps=1e-5), residual_mult=0.5,
+                layers=[dict(type="attention", mixer=mixer, mlp=mlp) for _ in range(L)])
+
+
 def design_run(args):
     """Decode at batch 1 / 8 / 64 (1024-token prompts) and one 2048-token prompt, for both designs of a shape."""
-    out = {"metric": f"decode and prefill tok/s, Pamopel beside Qwen3 at shape {args.design}, random weights",
+    out = {"metric": f"decode and prefill tok/s, designs beside Qwen3 at shape {args.design}, random weights",
            "unit": "tokens/s", "dtype": args.dtype, "data": "synthetic", "shape": args.design, "designs": {}}
-    for label, config in zip(("pamopel", "qwen3"), design_configs(args.design)):
-        if args.design_model not in ("both", label):
+    for label, config in zip(("pamopel", "qwen3", "ziferax"), design_configs(args.design) + (ziferax_config(args.design),)):
+        if args.design_model not in ("both", "all", label) or (label == "ziferax" and args.design_model == "both"):
             continue
         m = Sized(label, args.dtype, 4096, eager=args.eager, config=config)
         rec = {"weights_GB": round(m.wbytes / 1e9, 3), "decode": {}}

@@ -421,6 +421,33 @@ def test_router_scores_choice_and_weights(R, top, correction):
         assert (wts[t].double().cpu() - picked / (picked.sum() + 1e-20)).abs().max() < 1e-6
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H,R,top", [(40, 4, 4), (256, 20, 3), (2048, 36, 4), (100, 130, 8)])
+def test_router_product_and_routing_in_one_kernel(dtype, H, R, top):
+    """The fused kernel against the 64-bit product of the same (rounded) rows and the plain routing; a token's
+    choice and weights are the same bits whatever else is in the batch."""
+    from ullm_amd.kernels import ops
+    g = torch.Generator().manual_seed(H + R)
+    x = torch.randn(50, H, generator=g).to(dtype)
+    w = (torch.randn(R, H, generator=g) * 0.3).float()
+    c = (torch.randn(R, generator=g) * 0.1).float()
+    ids, wts = ops.moe_router(x.to(DEV), w.to(DEV), c.to(DEV), top)
+    one_ids, one_wts = ops.moe_router(x[17:18].to(DEV), w.to(DEV), c.to(DEV), top)
+    assert torch.equal(one_ids[0], ids[17]) and torch.equal(one_wts[0], wts[17])
+    s = torch.softmax(x.double() @ w.double().T, -1)
+    choice = s + c.double()
+    for t in range(50):
+        order = sorted(range(R), key=lambda e: (-float(choice[t, e]), e))
+        if top < R and float(choice[t, order[top - 1]] - choice[t, order[top]]) < 1e-5:
+            continue                                              # a close call: either choice is right
+        if min(float(choice[t, order[i]] - choice[t, order[i + 1]]) for i in range(top - 1)) < 1e-5 if top > 1 else False:
+            assert sorted(ids[t].tolist()) == sorted(order[:top])
+            continue
+        assert ids[t].tolist() == order[:top], t
+        picked = s[t, order[:top]]
+        assert (wts[t].double().cpu() - picked / (picked.sum() + 1e-20)).abs().max() < 1e-5
+
+
 @pytest.mark.parametrize("T,top,E,extra,rows", [(1, 3, 16, 4, 16), (7, 2, 3, 1, 16), (300, 4, 8, 0, 64), (129, 1, 40, 8, 32), (33, 8, 9, 3, 16)])
 def test_grouping_pairs_by_expert(T, top, E, extra, rows):
     from ullm_amd.kernels import ops
@@ -449,7 +476,8 @@ def test_grouping_pairs_by_expert(T, top, E, extra, rows):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("T,top,E,H,ff,rows", [(5, 2, 4, 64, 32, 16), (70, 3, 5, 136, 72, 16), (200, 2, 3, 128, 64, 64),
-                                               (90, 4, 6, 96, 40, 32), (9, 2, 3, 40, 12, 16), (3, 1, 2, 72, 8, 16)])
+                                               (90, 4, 6, 96, 40, 32), (9, 2, 3, 40, 12, 16), (3, 1, 2, 72, 8, 16),
+                                               (300, 3, 4, 200, 136, 64), (130, 2, 2, 72, 200, 64)])
 def test_expert_products_over_grouped_rows_and_their_weighted_sum(dtype, T, top, E, H, ff, rows):
     """gate | up with the clamped unit, down, and the sum with identity experts, a shared branch, another branch and a
     bias, against 64-bit products of the same operands; sizes the matrix-core tiles take and sizes they do not (an

@@ -32,29 +32,28 @@ union Pack8 {
 #define MOE_MAX_TOP 32
 
 // ------------------------------------------------------------------------------- routing
-__global__ void __launch_bounds__(64)
-moe_route_kernel(const float* __restrict__ logits, int ld, const float* __restrict__ correction, int n_router, int top,
-                 int* __restrict__ ids, float* __restrict__ weights) {
-  __shared__ float s_soft[MOE_MAX_ROUTER], s_choice[MOE_MAX_ROUTER];
-  __shared__ float s_pick[MOE_MAX_TOP];
-  const int t = blockIdx.x, lane = threadIdx.x;
-  const float* z = logits + (size_t)t * ld;
+// One wave: softmax over the logits z[0 .. n_router) in shared memory (overwritten by the scores), the `top` largest
+// of score + correction, the chosen scores over their sum.  s_choice holds n_router floats, s_pick MOE_MAX_TOP.
+__device__ __forceinline__ void route_from_logits(float* z, float* s_choice, float* s_pick,
+                                                  const float* __restrict__ correction, int n_router, int top,
+                                                  int* __restrict__ ids, float* __restrict__ weights, int lane) {
   float mx = -INFINITY;
   for (int e = lane; e < n_router; e += 64) mx = fmaxf(mx, z[e]);
   mx = wave_max(mx);
   float sum = 0.f;
   for (int e = lane; e < n_router; e += 64) {
     const float p = expf(z[e] - mx);
-    s_soft[e] = p;
+    z[e] = p;
     sum += p;
   }
   sum = wave_sum(sum);
   for (int e = lane; e < n_router; e += 64) {
-    const float s = s_soft[e] / sum;
-    s_soft[e] = s;
+    const float s = z[e] / sum;
+    z[e] = s;
     s_choice[e] = s + (correction ? correction[e] : 0.f);
   }
-  __syncthreads();
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __builtin_amdgcn_wave_barrier();
   float total = 0.f;
   for (int k = 0; k < top; ++k) {
     float best = -INFINITY;
@@ -76,16 +75,28 @@ moe_route_kernel(const float* __restrict__ logits, int ld, const float* __restri
       }
     }
     if (at >= n_router) at = k < n_router ? k : 0;       // every value a NaN: any expert
-    const float s = s_soft[at];
+    const float s = z[at];
     total += s;
     if (lane == 0) {
-      ids[(size_t)t * top + k] = at;
+      ids[k] = at;
       s_pick[k] = s;
       s_choice[at] = -INFINITY;
     }
-    __syncthreads();
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_wave_barrier();
   }
-  if (lane < top) weights[(size_t)t * top + lane] = s_pick[lane] / (total + 1e-20f);
+  if (lane < top) weights[lane] = s_pick[lane] / (total + 1e-20f);
+}
+
+__global__ void __launch_bounds__(64)
+moe_route_kernel(const float* __restrict__ logits, int ld, const float* __restrict__ correction, int n_router, int top,
+                 int* __restrict__ ids, float* __restrict__ weights) {
+  __shared__ float s_soft[MOE_MAX_ROUTER], s_choice[MOE_MAX_ROUTER];
+  __shared__ float s_pick[MOE_MAX_TOP];
+  const int t = blockIdx.x, lane = threadIdx.x;
+  for (int e = lane; e < n_router; e += 64) s_soft[e] = logits[(size_t)t * ld + e];
+  __syncthreads();
+  route_from_logits(s_soft, s_choice, s_pick, correction, n_router, top, ids + (size_t)t * top, weights + (size_t)t * top, lane);
 }
 
 extern "C" int ullm_moe_route(const float* logits, int ld, const float* correction, int T_, int n_router, int top,
@@ -94,6 +105,50 @@ extern "C" int ullm_moe_route(const float* logits, int ld, const float* correcti
   if (n_router < 1 || n_router > MOE_MAX_ROUTER || top < 1 || top > MOE_MAX_TOP || top > n_router || ld < n_router)
     return ULLM_ERR_SHAPE;
   hipLaunchKernelGGL(moe_route_kernel, dim3(T_), dim3(64), 0, stream, logits, ld, correction, n_router, top, ids, weights);
+  ULLM_LAUNCH_CHECK();
+}
+
+// The router's product and the routing in one kernel: a block per token; the token's row in shared memory as 32-bit
+// values, every wave takes router outputs in turn (lanes stride the row, then the wave adds up: an order that depends
+// on nothing but the row), the first wave routes.  The router's matrix is 32-bit [n_router, H].
+template <typename T>
+__global__ void __launch_bounds__(256)
+moe_router_kernel(const T* __restrict__ x, int ldx, const float* __restrict__ w, const float* __restrict__ correction,
+                  int H, int n_router, int top, int* __restrict__ ids, float* __restrict__ weights) {
+  extern __shared__ float xrow[];
+  __shared__ float z[MOE_MAX_ROUTER], s_choice[MOE_MAX_ROUTER];
+  __shared__ float s_pick[MOE_MAX_TOP];
+  const int t = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const T* xr = x + (size_t)t * ldx;
+  for (int i = tid; i < H; i += 256) xrow[i] = ld_f32(xr + i);
+  __syncthreads();
+  for (int e = wave; e < n_router; e += 4) {
+    const float* we = w + (size_t)e * H;
+    float a = 0.f;
+    for (int i = lane; i < H; i += 64) a = fmaf(xrow[i], we[i], a);
+    a = wave_sum(a);
+    if (lane == 0) z[e] = a;
+  }
+  __syncthreads();
+  if (wave == 0)
+    route_from_logits(z, s_choice, s_pick, correction, n_router, top, ids + (size_t)t * top, weights + (size_t)t * top, lane);
+}
+
+extern "C" int ullm_moe_router(const void* x, int ldx, const float* w, const float* correction, int T_, int H,
+                               int n_router, int top, int* ids, float* weights, int dtype, hipStream_t stream) {
+  if (T_ <= 0) return 0;
+  if (n_router < 1 || n_router > MOE_MAX_ROUTER || top < 1 || top > MOE_MAX_TOP || top > n_router || H < 1 || ldx < H ||
+      (size_t)H * sizeof(float) > 48 * 1024)
+    return ULLM_ERR_SHAPE;
+  const size_t lds = (size_t)H * sizeof(float);
+  if (dtype == ULLM_F32)
+    hipLaunchKernelGGL(moe_router_kernel<float>, dim3(T_), dim3(256), lds, stream, (const float*)x, ldx, w, correction, H,
+                       n_router, top, ids, weights);
+  else if (dtype == ULLM_BF16)
+    hipLaunchKernelGGL(moe_router_kernel<bf16_t>, dim3(T_), dim3(256), lds, stream, (const bf16_t*)x, ldx, w, correction, H,
+                       n_router, top, ids, weights);
+  else
+    return ULLM_ERR_DTYPE;
   ULLM_LAUNCH_CHECK();
 }
 
@@ -214,20 +269,24 @@ moe_rows_simple_kernel(const T* __restrict__ x, int ldx, const int* __restrict__
 }
 
 // ------------------------------------------------------------------------------- products on the matrix cores
-// grid (tiles, column blocks); tile = up to 16 * MT grouped rows of one expert; a block's WAVES waves take 16
-// output columns each (GATED: the 16 gate rows and the 16 up rows of those columns) over all of K, two steps of 32
-// in flight.  No load stands under a condition: a row past the tile's reads its last row, a column past the end
-// the last column, a piece past the end of K the row's last piece (and is replaced by zeros); none is stored.
+// Few rows a tile (single tokens of a step): grid (tiles, groups of 16 output columns); tile = up to 16 * MT grouped
+// rows of one expert.  The block's four waves share the 16 columns (GATED: the 16 gate rows and the 16 up rows of
+// those columns) and take every fourth step of 64 along K, two steps of 32 in flight each; their sums are added
+// through shared memory in wave order.  The work is streaming the chosen experts' matrices once, so it is cut into
+// many blocks with many loads under way.  No load stands under a condition: a row past the tile's reads its last
+// row, a column past the end the last column, a piece past the end of K the row's last piece (and is replaced by
+// zeros); none is stored.
 template <int MT, bool GATED>
 __global__ void __launch_bounds__(256)
 moe_rows_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const int* __restrict__ row_index,
                      const bf16_t* __restrict__ w, const int* __restrict__ tiles, void* __restrict__ out_, int ldo,
                      int n_out, int K, float limit, float alpha) {
+  constexpr int VALS = (GATED ? 8 : 4) * MT;
+  __shared__ float part[3][VALS][64];
   const int tile = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 15, g = lane >> 4;
   const int e = tiles[3 * tile], slot0 = tiles[3 * tile + 1], rows = tiles[3 * tile + 2];
   if (rows <= 0) return;
-  const int n0 = (blockIdx.y * 4 + wave) * 16;
-  if (n0 >= n_out) return;
+  const int n0 = blockIdx.y * 16;
   const size_t w_rows = GATED ? 2 * (size_t)n_out : (size_t)n_out;
   const int wrow = n0 + r < n_out ? n0 + r : n_out - 1;
   const bf16_t* wg = w + ((size_t)e * w_rows + wrow) * K;
@@ -246,7 +305,7 @@ moe_rows_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const int* __restric
   }
   const int last_piece = K - 8;                          // K is a multiple of 8
   const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
-  for (int k0 = 0; k0 < K; k0 += 64) {
+  for (int k0 = 64 * wave; k0 < K; k0 += 256) {
     Pack8 a_g[2], a_u[2], b[2][MT];
     bool in[2];
 #pragma unroll
@@ -269,6 +328,27 @@ moe_rows_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const int* __restric
       }
     }
   }
+  // the waves' sums, added in wave order
+  if (wave > 0) {
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        part[wave - 1][(GATED ? 8 : 4) * t + i][lane] = acc_g[t][i];
+        if (GATED) part[wave - 1][8 * t + 4 + i][lane] = acc_u[t][i];
+      }
+  }
+  __syncthreads();
+  if (wave > 0) return;
+#pragma unroll
+  for (int v = 0; v < 3; ++v)
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        acc_g[t][i] += part[v][(GATED ? 8 : 4) * t + i][lane];
+        if (GATED) acc_u[t][i] += part[v][8 * t + 4 + i][lane];
+      }
   // lane (r, g): row r of each 16-row group, columns n0 + 4g .. + 4
   const int c = n0 + 4 * g;
 #pragma unroll
@@ -301,6 +381,130 @@ moe_rows_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const int* __restric
   }
 }
 
+// Many rows a tile (prompt portions): grid (tiles, blocks of 128 rows of the expert's matrix); tile = up to 64 grouped
+// rows of one expert.  A stage is 64 values of K: the tile's 64 rows of x and 128 rows of the matrix (GATED: the
+// gate rows and the up rows of 64 output columns; else 128 output columns) go through shared memory once a block,
+// 128-byte rows whose 16-byte piece c of row r lies at piece c ^ ((r >> 1) & 7) (the 16 lanes the hardware serves
+// together then read 16 different bank groups); the next stage is fetched into registers while the products of this
+// one run.  Wave v takes matrix rows 16 v .. and 64 + 16 v .. (GATED: gate and up of the same columns) against all
+// 64 rows of x: 16 products per 12 reads of shared memory.
+template <bool GATED>
+__global__ void __launch_bounds__(256)
+moe_tiles_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const int* __restrict__ row_index,
+                      const bf16_t* __restrict__ w, const int* __restrict__ tiles, void* __restrict__ out_, int ldo,
+                      int n_out, int K, float limit, float alpha) {
+  __shared__ __attribute__((aligned(16))) unsigned char xs[64 * 128];
+  __shared__ __attribute__((aligned(16))) unsigned char ws[128 * 128];
+  const int tile = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 15, g = lane >> 4;
+  const int e = tiles[3 * tile], slot0 = tiles[3 * tile + 1], rows = tiles[3 * tile + 2];
+  if (rows <= 0) return;
+  const int cols = GATED ? 64 : 128;                      // output columns of a block
+  const int n0 = blockIdx.y * cols;
+  const size_t w_rows = GATED ? 2 * (size_t)n_out : (size_t)n_out;
+  const bf16_t* we = w + (size_t)e * w_rows * K;
+  // what this thread fetches of a stage: piece `pc` of x rows prow, prow + 32 and of matrix rows prow + 32 i
+  const int pc = tid & 7, prow = tid >> 3;
+  const bf16_t* xsrc[2];
+  const bf16_t* wsrc[4];
+  int xput[2], wput[4];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int row = prow + 32 * i, rr = row < rows ? row : rows - 1;
+    xsrc[i] = x + (size_t)(row_index ? row_index[slot0 + rr] : slot0 + rr) * ldx;
+    xput[i] = row * 128 + ((pc ^ ((row >> 1) & 7)) << 4);
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int row = prow + 32 * i;                       // 0 .. 127 of the block's matrix rows
+    int n = GATED ? n0 + (row & 63) : n0 + row;
+    if (n >= n_out) n = n_out - 1;
+    wsrc[i] = we + ((GATED && row >= 64 ? (size_t)n_out : 0) + n) * K;
+    wput[i] = row * 128 + ((pc ^ ((row >> 1) & 7)) << 4);
+  }
+  const int last_piece = K - 8;
+  const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+  uint4 xreg[2], wreg[4];
+  auto fetch = [&](int k0) __attribute__((always_inline)) {
+    const int k = k0 + 8 * pc;
+    const bool in = k <= last_piece;
+    const int kk = in ? k : last_piece;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) xreg[i] = ld16(xsrc[i] + kk);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) wreg[i] = ld_stream16(wsrc[i] + kk);
+    if (!in) {
+#pragma unroll
+      for (int i = 0; i < 2; ++i) xreg[i] = zero;
+    }
+  };
+  f32x4_t acc[2][4];
+#pragma unroll
+  for (int h = 0; h < 2; ++h)
+#pragma unroll
+    for (int t = 0; t < 4; ++t) acc[h][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  fetch(0);
+  for (int k0 = 0; k0 < K; k0 += 64) {
+    __syncthreads();                                      // the products of the stage before are done
+#pragma unroll
+    for (int i = 0; i < 2; ++i) st16(xs + xput[i], xreg[i]);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) st16(ws + wput[i], wreg[i]);
+    __syncthreads();
+    if (k0 + 64 < K) fetch(k0 + 64);
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      Pack8 a[2], b[4];
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int row = 64 * h + 16 * wave + r;
+        a[h].u4 = ld16(ws + row * 128 + (((4 * s + g) ^ ((row >> 1) & 7)) << 4));
+      }
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const int row = 16 * t + r;
+        b[t].u4 = ld16(xs + row * 128 + (((4 * s + g) ^ ((row >> 1) & 7)) << 4));
+      }
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) acc[h][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[h].v, b[t].v, acc[h][t], 0, 0, 0);
+    }
+  }
+  // lane (r, g): row r of each 16-row group; columns 16 wave + 4g .. + 4 of the block's (and 64 further on)
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    const int row = 16 * t + r;
+    if (row >= rows) continue;
+    if (GATED) {
+      const int c = n0 + 16 * wave + 4 * g;
+      bf16_t* o = reinterpret_cast<bf16_t*>(out_) + (size_t)(slot0 + row) * ldo + c;
+      float v[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = moe_glu<false>(acc[0][t][i], acc[1][t][i], limit, alpha);
+      if (c + 3 < n_out && (ldo & 3) == 0) {
+        *reinterpret_cast<uint2*>(o) = make_uint2(pack2_bf16(v[0], v[1]), pack2_bf16(v[2], v[3]));
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (c + i < n_out) o[i] = f32_to_bf16_bits(v[i]);
+      }
+    } else {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int c = n0 + 64 * h + 16 * wave + 4 * g;
+        float* o = reinterpret_cast<float*>(out_) + (size_t)(slot0 + row) * ldo + c;
+        if (c + 3 < n_out && (ldo & 3) == 0) {
+          *reinterpret_cast<float4*>(o) = make_float4(acc[h][t][0], acc[h][t][1], acc[h][t][2], acc[h][t][3]);
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (c + i < n_out) o[i] = acc[h][t][i];
+        }
+      }
+    }
+  }
+}
+
 // Rows of a tile the matrix-core kernels take for a launch made with `tile_rows` rows a tile.
 extern "C" int ullm_moe_mfma_supports(int K, int ldx, int tile_rows) {
   return K >= 8 && K % 8 == 0 && ldx % 8 == 0 && (tile_rows == 16 || tile_rows == 32 || tile_rows == 64);
@@ -314,13 +518,23 @@ extern "C" int ullm_moe_rows(const void* x, int ldx, const int* row_index, const
   if (max_tiles <= 0) return 0;
   if (n_out < 1 || K < 1 || ldx < K || ldo < n_out || tile_rows < 1) return ULLM_ERR_SHAPE;
   if (dtype == ULLM_BF16 && ullm_moe_mfma_supports(K, ldx, tile_rows) && !((uintptr_t)x & 15) && !((uintptr_t)w & 15)) {
-    dim3 grid(max_tiles, (n_out + 63) / 64), block(256);
+    if (tile_rows == 64) {
+      dim3 grid(max_tiles, (n_out + (gated ? 63 : 127)) / (gated ? 64 : 128)), block(256);
+      if (grid.y > 65535) return ULLM_ERR_SHAPE;
+      if (gated)
+        hipLaunchKernelGGL(moe_tiles_mfma_kernel<true>, grid, block, 0, stream, (const bf16_t*)x, ldx, row_index,
+                           (const bf16_t*)w, tiles, out, ldo, n_out, K, limit, alpha);
+      else
+        hipLaunchKernelGGL(moe_tiles_mfma_kernel<false>, grid, block, 0, stream, (const bf16_t*)x, ldx, row_index,
+                           (const bf16_t*)w, tiles, out, ldo, n_out, K, limit, alpha);
+      ULLM_LAUNCH_CHECK();
+    }
+    dim3 grid(max_tiles, (n_out + 15) / 16), block(256);
     if (grid.y > 65535) return ULLM_ERR_SHAPE;
 #define GO(MT, G) hipLaunchKernelGGL((moe_rows_mfma_kernel<MT, G>), grid, block, 0, stream, (const bf16_t*)x, ldx, row_index, \
     (const bf16_t*)w, tiles, out, ldo, n_out, K, limit, alpha)
     if (tile_rows == 16) { if (gated) GO(1, true); else GO(1, false); }
-    else if (tile_rows == 32) { if (gated) GO(2, true); else GO(2, false); }
-    else { if (gated) GO(4, true); else GO(4, false); }
+    else { if (gated) GO(2, true); else GO(2, false); }
 #undef GO
     ULLM_LAUNCH_CHECK();
   }
@@ -340,26 +554,37 @@ extern "C" int ullm_moe_rows(const void* x, int ldx, const int* row_index, const
 
 // ------------------------------------------------------------------------------- the weighted sum
 // out[t][c] = base[t][c] + bias[c] + shared[t][c] + sum_k weights[t][k] * (ids[t][k] < n_experts ? y[slot][c] : x[t][c]);
-// base (float32 or TX), bias (float32), shared (TX) may be null.  Four columns a thread where rows allow.
-template <typename TX, typename TB>
+// base (float32 or TX), bias (float32), shared (TX) may be null.  grid (tokens, groups of columns): a thread takes
+// VEC consecutive columns, all its loads independent of each other.
+template <typename TX, typename TB, int VEC>
 __global__ void __launch_bounds__(256)
 moe_combine_kernel(const float* __restrict__ y, const TX* __restrict__ x, int ldx, const int* __restrict__ ids,
                    const float* __restrict__ weights, const int* __restrict__ slot_of_pair, int top, int n_experts,
                    const TB* __restrict__ base, const float* __restrict__ bias, const TX* __restrict__ shared,
                    float* __restrict__ out, int H) {
-  const int t = blockIdx.x;
-  for (int c = threadIdx.x; c < H; c += 256) {
-    float a = base ? ld_f32(base + (size_t)t * H + c) : 0.f;
-    if (bias) a += bias[c];
-    if (shared) a += ld_f32(shared + (size_t)t * H + c);
-    for (int k = 0; k < top; ++k) {
-      const int e = ids[(size_t)t * top + k];
-      const float wk = weights[(size_t)t * top + k];
-      const float v = e < n_experts ? y[(size_t)slot_of_pair[(size_t)t * top + k] * H + c] : ld_f32(x + (size_t)t * ldx + c);
-      a = fmaf(wk, v, a);
-    }
-    out[(size_t)t * H + c] = a;
+  const int t = blockIdx.x, c = VEC * (blockIdx.y * 256 + threadIdx.x);
+  if (c >= H) return;
+  float a[VEC];
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) {
+    a[i] = base ? ld_f32(base + (size_t)t * H + c + i) : 0.f;
+    if (bias) a[i] += bias[c + i];
+    if (shared) a[i] += ld_f32(shared + (size_t)t * H + c + i);
   }
+  for (int k = 0; k < top; ++k) {
+    const int e = ids[(size_t)t * top + k];
+    const float wk = weights[(size_t)t * top + k];
+    if (e < n_experts) {
+      const float* yr = y + (size_t)slot_of_pair[(size_t)t * top + k] * H + c;
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) a[i] = fmaf(wk, yr[i], a[i]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) a[i] = fmaf(wk, ld_f32(x + (size_t)t * ldx + c + i), a[i]);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) out[(size_t)t * H + c + i] = a[i];
 }
 
 extern "C" int ullm_moe_combine(const float* y, const void* x, int ldx, const int* ids, const float* weights,
@@ -368,18 +593,22 @@ extern "C" int ullm_moe_combine(const float* y, const void* x, int ldx, const in
                                 hipStream_t stream) {
   if (T_ <= 0) return 0;
   if (H < 1 || top < 1 || ldx < H) return ULLM_ERR_SHAPE;
-  dim3 grid(T_), block(256);
-#define GO(TX, TB) hipLaunchKernelGGL((moe_combine_kernel<TX, TB>), grid, block, 0, stream, y, (const TX*)x, ldx, ids, weights, \
+  const int vec = H % 4 == 0 ? 4 : 1;
+  dim3 grid(T_, (H / vec + 255) / 256), block(256);
+  if (grid.y > 65535) return ULLM_ERR_SHAPE;
+#define GO(TX, TB, V) hipLaunchKernelGGL((moe_combine_kernel<TX, TB, V>), grid, block, 0, stream, y, (const TX*)x, ldx, ids, weights, \
     slot_of_pair, top, n_experts, (const TB*)base, bias, (const TX*)shared, out, H)
+#define GOV(TX, TB) do { if (vec == 4) GO(TX, TB, 4); else GO(TX, TB, 1); } while (0)
   if (dtype == ULLM_F32) {
     if (base && base_dtype != ULLM_F32) return ULLM_ERR_DTYPE;
-    GO(float, float);
+    GOV(float, float);
   } else if (dtype == ULLM_BF16) {
-    if (base && base_dtype == ULLM_BF16) GO(bf16_t, bf16_t);
-    else GO(bf16_t, float);
+    if (base && base_dtype == ULLM_BF16) GOV(bf16_t, bf16_t);
+    else GOV(bf16_t, float);
   } else {
     return ULLM_ERR_DTYPE;
   }
+#undef GOV
 #undef GO
   ULLM_LAUNCH_CHECK();
 }

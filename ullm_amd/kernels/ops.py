@@ -1071,6 +1071,30 @@ def moe_route(logits: torch.Tensor, correction: Optional[torch.Tensor], top: int
     return ids, weights
 
 
+MOE_ROUTER_MAX_WIDTH = 12288      # widest row the fused router kernel keeps in shared memory
+
+
+def moe_router(x: torch.Tensor, w_router: torch.Tensor, correction: Optional[torch.Tensor], top: int):
+    """:func:`moe_route` of the 32-bit product of ``x`` [T, H] with ``w_router`` (float32 [R, H]), in one kernel: every
+    router output is summed along the row in an order that depends on nothing but the row."""
+    T, H = x.shape
+    R = w_router.shape[0]
+    _need(x.stride(1) == 1 and H <= MOE_ROUTER_MAX_WIDTH, f"x must be [T, H <= {MOE_ROUTER_MAX_WIDTH}] with unit stride")
+    _need(w_router.dtype == torch.float32 and w_router.shape == (R, H) and w_router.is_contiguous(),
+          "the router's matrix must be contiguous float32 [R, H]")
+    _need(1 <= top <= min(R, MOE_MAX_TOP) and R <= MOE_MAX_ROUTER, f"top {top} of {R} router outputs: at most "
+          f"{MOE_MAX_TOP} of {MOE_MAX_ROUTER}")
+    if correction is not None:
+        _need(correction.dtype == torch.float32 and correction.numel() == R and correction.is_contiguous(),
+              "the router's correction must be float32 [R]")
+    ids = torch.empty((T, top), dtype=torch.int32, device=x.device)
+    weights = torch.empty((T, top), dtype=torch.float32, device=x.device)
+    _check(build.load("moe").ullm_moe_router(_p(x), _c_int(x.stride(0)), _p(w_router), _p(correction), _c_int(T), _c_int(H),
+                                             _c_int(R), _c_int(top), _p(ids), _p(weights), _c_int(_dt(x)), _stream()),
+           "moe_router")
+    return ids, weights
+
+
 def moe_max_tiles(n_pairs: int, n_experts: int, tile_rows: int) -> int:
     """The most tiles of ``tile_rows`` rows that ``n_pairs`` (token, expert) pairs over ``n_experts`` experts can fill."""
     return max(1, n_pairs // tile_rows + min(n_experts, n_pairs))

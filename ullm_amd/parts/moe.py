@@ -95,6 +95,8 @@ class RoutedExperts(FeedForward):
     # ------------------------------------------------------------------ the step
     def route(self, x: torch.Tensor):
         """(ids int32 [T, top], weights float32 [T, top]) of the rows of x."""
+        if self.hidden_size <= ops.MOE_ROUTER_MAX_WIDTH:
+            return ops.moe_router(x, self.w_router, self.correction, self.top)     # the product and the routing in one
         logits = ops.gemm_simple(x, self.w_router, out_dtype=torch.float32)       # 32-bit sums in a fixed order
         return ops.moe_route(logits, self.correction, self.top)
 
