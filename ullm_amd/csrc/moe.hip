@@ -115,19 +115,51 @@ template <typename T>
 __global__ void __launch_bounds__(256)
 moe_router_kernel(const T* __restrict__ x, int ldx, const float* __restrict__ w, const float* __restrict__ correction,
                   int H, int n_router, int top, int* __restrict__ ids, float* __restrict__ weights) {
-  extern __shared__ float xrow[];
+  extern __shared__ __attribute__((aligned(16))) float xrow[];
   __shared__ float z[MOE_MAX_ROUTER], s_choice[MOE_MAX_ROUTER];
   __shared__ float s_pick[MOE_MAX_TOP];
   const int t = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const T* xr = x + (size_t)t * ldx;
   for (int i = tid; i < H; i += 256) xrow[i] = ld_f32(xr + i);
   __syncthreads();
-  for (int e = wave; e < n_router; e += 4) {
-    const float* we = w + (size_t)e * H;
-    float a = 0.f;
-    for (int i = lane; i < H; i += 64) a = fmaf(xrow[i], we[i], a);
-    a = wave_sum(a);
-    if (lane == 0) z[e] = a;
+  // four router outputs a wave at a time, four 16-byte pieces of each row a lane under way: the loop is a chain of
+  // trips to memory otherwise.  A lane adds its pieces in rising order, then the wave adds up.
+  const bool vec = (H & 3) == 0 && (((uintptr_t)w) & 15) == 0;
+  for (int e0 = 4 * wave; e0 < n_router; e0 += 16) {
+    float a[4] = {0.f, 0.f, 0.f, 0.f};
+    const float* we[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) we[u] = w + (size_t)(e0 + u < n_router ? e0 + u : n_router - 1) * H;
+    if (vec) {
+      const int pieces = H >> 2;
+      for (int p0 = lane; p0 < pieces; p0 += 256) {
+        float4 wv[4][4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int pj = p0 + 64 * j < pieces ? p0 + 64 * j : pieces - 1;
+#pragma unroll
+          for (int u = 0; u < 4; ++u) wv[u][j] = *reinterpret_cast<const float4*>(we[u] + 4 * pj);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          if (p0 + 64 * j >= pieces) break;
+          const float4 xv = *reinterpret_cast<const float4*>(xrow + 4 * (p0 + 64 * j));
+#pragma unroll
+          for (int u = 0; u < 4; ++u)
+            a[u] = fmaf(xv.w, wv[u][j].w, fmaf(xv.z, wv[u][j].z, fmaf(xv.y, wv[u][j].y, fmaf(xv.x, wv[u][j].x, a[u]))));
+        }
+      }
+    } else {
+      for (int i = lane; i < H; i += 64) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) a[u] = fmaf(xrow[i], we[u][i], a[u]);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const float sum = wave_sum(a[u]);
+      if (lane == 0 && e0 + u < n_router) z[e0 + u] = sum;
+    }
   }
   __syncthreads();
   if (wave == 0)
@@ -393,8 +425,8 @@ __global__ void __launch_bounds__(256)
 moe_tiles_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const int* __restrict__ row_index,
                       const bf16_t* __restrict__ w, const int* __restrict__ tiles, void* __restrict__ out_, int ldo,
                       int n_out, int K, float limit, float alpha) {
-  __shared__ __attribute__((aligned(16))) unsigned char xs[64 * 128];
-  __shared__ __attribute__((aligned(16))) unsigned char ws[128 * 128];
+  __shared__ __attribute__((aligned(16))) unsigned char xs2[2][64 * 128];      // two stages take turns
+  __shared__ __attribute__((aligned(16))) unsigned char ws2[2][128 * 128];
   const int tile = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 15, g = lane >> 4;
   const int e = tiles[3 * tile], slot0 = tiles[3 * tile + 1], rows = tiles[3 * tile + 2];
   if (rows <= 0) return;
@@ -442,15 +474,21 @@ moe_tiles_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const int* __restri
   for (int h = 0; h < 2; ++h)
 #pragma unroll
     for (int t = 0; t < 4; ++t) acc[h][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  auto put = [&](int buf) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) st16(xs2[buf] + xput[i], xreg[i]);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) st16(ws2[buf] + wput[i], wreg[i]);
+  };
   fetch(0);
-  for (int k0 = 0; k0 < K; k0 += 64) {
-    __syncthreads();                                      // the products of the stage before are done
-#pragma unroll
-    for (int i = 0; i < 2; ++i) st16(xs + xput[i], xreg[i]);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) st16(ws + wput[i], wreg[i]);
-    __syncthreads();
-    if (k0 + 64 < K) fetch(k0 + 64);
+  put(0);
+  __syncthreads();
+  int cur = 0;
+  for (int k0 = 0; k0 < K; k0 += 64, cur ^= 1) {
+    const bool more = k0 + 64 < K;
+    if (more) fetch(k0 + 64);                             // on its way while this stage's products run
+    const unsigned char* xs = xs2[cur];
+    const unsigned char* ws = ws2[cur];
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
       Pack8 a[2], b[4];
@@ -469,6 +507,9 @@ moe_tiles_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const int* __restri
 #pragma unroll
         for (int t = 0; t < 4; ++t) acc[h][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[h].v, b[t].v, acc[h][t], 0, 0, 0);
     }
+    // the other stage was last read before the barrier that ended the step before: it can be written now
+    if (more) put(cur ^ 1);
+    __syncthreads();
   }
   // lane (r, g): row r of each 16-row group; columns 16 wave + 4g .. + 4 of the block's (and 64 further on)
 #pragma unroll
