@@ -434,6 +434,10 @@ def test_router_product_and_routing_in_one_kernel(dtype, H, R, top):
     ids, wts = ops.moe_router(x.to(DEV), w.to(DEV), c.to(DEV), top)
     one_ids, one_wts = ops.moe_router(x[17:18].to(DEV), w.to(DEV), c.to(DEV), top)
     assert torch.equal(one_ids[0], ids[17]) and torch.equal(one_wts[0], wts[17])
+    # many tokens take the variant with four tokens a block: the same bits again
+    many = torch.cat([x] * 13)[:-3]
+    many_ids, many_wts = ops.moe_router(many.to(DEV), w.to(DEV), c.to(DEV), top)
+    assert torch.equal(many_ids[:50], ids) and torch.equal(many_wts[600:], wts[:47]) and torch.equal(many_wts[:50], wts)
     s = torch.softmax(x.double() @ w.double().T, -1)
     choice = s + c.double()
     for t in range(50):

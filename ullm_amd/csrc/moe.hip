@@ -108,25 +108,33 @@ extern "C" int ullm_moe_route(const float* logits, int ld, const float* correcti
   ULLM_LAUNCH_CHECK();
 }
 
-// The router's product and the routing in one kernel: a block per token; the token's row in shared memory as 32-bit
-// values, every wave takes router outputs in turn (lanes stride the row, then the wave adds up: an order that depends
-// on nothing but the row), the first wave routes.  The router's matrix is 32-bit [n_router, H].
-template <typename T>
+// The router's product and the routing in one kernel: a block takes TPB tokens; their rows lie in shared memory as
+// 32-bit values, every wave takes four router outputs at a time with four 16-byte pieces of each of their rows a
+// lane under way (the loop is a chain of trips to memory otherwise), and every piece fetched serves all the block's
+// tokens.  A lane adds a token's pieces in rising order, then the wave adds up: an order that depends on nothing but
+// the row.  Then wave v routes token v.  The router's matrix is 32-bit [n_router, H].
+template <typename T, int TPB>
 __global__ void __launch_bounds__(256)
 moe_router_kernel(const T* __restrict__ x, int ldx, const float* __restrict__ w, const float* __restrict__ correction,
-                  int H, int n_router, int top, int* __restrict__ ids, float* __restrict__ weights) {
-  extern __shared__ __attribute__((aligned(16))) float xrow[];
-  __shared__ float z[MOE_MAX_ROUTER], s_choice[MOE_MAX_ROUTER];
-  __shared__ float s_pick[MOE_MAX_TOP];
-  const int t = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const T* xr = x + (size_t)t * ldx;
-  for (int i = tid; i < H; i += 256) xrow[i] = ld_f32(xr + i);
+                  int n_tokens, int H, int n_router, int top, int* __restrict__ ids, float* __restrict__ weights) {
+  extern __shared__ __attribute__((aligned(16))) float xrow[];          // [TPB][H]
+  constexpr int RCAP = TPB == 1 ? MOE_MAX_ROUTER : 256;                // router outputs the variant takes
+  __shared__ float z[TPB][RCAP], s_choice[TPB][RCAP];
+  __shared__ float s_pick[TPB][MOE_MAX_TOP];
+  const int t0 = blockIdx.x * TPB, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+#pragma unroll
+  for (int q = 0; q < TPB; ++q) {
+    const T* xr = x + (size_t)(t0 + q < n_tokens ? t0 + q : n_tokens - 1) * ldx;
+    for (int i = tid; i < H; i += 256) xrow[q * H + i] = ld_f32(xr + i);
+  }
   __syncthreads();
-  // four router outputs a wave at a time, four 16-byte pieces of each row a lane under way: the loop is a chain of
-  // trips to memory otherwise.  A lane adds its pieces in rising order, then the wave adds up.
   const bool vec = (H & 3) == 0 && (((uintptr_t)w) & 15) == 0;
   for (int e0 = 4 * wave; e0 < n_router; e0 += 16) {
-    float a[4] = {0.f, 0.f, 0.f, 0.f};
+    float a[TPB][4];
+#pragma unroll
+    for (int q = 0; q < TPB; ++q)
+#pragma unroll
+      for (int u = 0; u < 4; ++u) a[q][u] = 0.f;
     const float* we[4];
 #pragma unroll
     for (int u = 0; u < 4; ++u) we[u] = w + (size_t)(e0 + u < n_router ? e0 + u : n_router - 1) * H;
@@ -143,27 +151,35 @@ moe_router_kernel(const T* __restrict__ x, int ldx, const float* __restrict__ w,
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           if (p0 + 64 * j >= pieces) break;
-          const float4 xv = *reinterpret_cast<const float4*>(xrow + 4 * (p0 + 64 * j));
 #pragma unroll
-          for (int u = 0; u < 4; ++u)
-            a[u] = fmaf(xv.w, wv[u][j].w, fmaf(xv.z, wv[u][j].z, fmaf(xv.y, wv[u][j].y, fmaf(xv.x, wv[u][j].x, a[u]))));
+          for (int q = 0; q < TPB; ++q) {
+            const float4 xv = *reinterpret_cast<const float4*>(xrow + q * H + 4 * (p0 + 64 * j));
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+              a[q][u] = fmaf(xv.w, wv[u][j].w, fmaf(xv.z, wv[u][j].z, fmaf(xv.y, wv[u][j].y, fmaf(xv.x, wv[u][j].x, a[q][u]))));
+          }
         }
       }
     } else {
       for (int i = lane; i < H; i += 64) {
 #pragma unroll
-        for (int u = 0; u < 4; ++u) a[u] = fmaf(xrow[i], we[u][i], a[u]);
+        for (int q = 0; q < TPB; ++q)
+#pragma unroll
+          for (int u = 0; u < 4; ++u) a[q][u] = fmaf(xrow[q * H + i], we[u][i], a[q][u]);
       }
     }
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const float sum = wave_sum(a[u]);
-      if (lane == 0 && e0 + u < n_router) z[e0 + u] = sum;
-    }
+    for (int q = 0; q < TPB; ++q)
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const float sum = wave_sum(a[q][u]);
+        if (lane == 0 && e0 + u < n_router) z[q][e0 + u] = sum;
+      }
   }
   __syncthreads();
-  if (wave == 0)
-    route_from_logits(z, s_choice, s_pick, correction, n_router, top, ids + (size_t)t * top, weights + (size_t)t * top, lane);
+  if (wave < TPB && t0 + wave < n_tokens)
+    route_from_logits(z[wave], s_choice[wave], s_pick[wave], correction, n_router, top, ids + (size_t)(t0 + wave) * top,
+                      weights + (size_t)(t0 + wave) * top, lane);
 }
 
 extern "C" int ullm_moe_router(const void* x, int ldx, const float* w, const float* correction, int T_, int H,
@@ -172,15 +188,17 @@ extern "C" int ullm_moe_router(const void* x, int ldx, const float* w, const flo
   if (n_router < 1 || n_router > MOE_MAX_ROUTER || top < 1 || top > MOE_MAX_TOP || top > n_router || H < 1 || ldx < H ||
       (size_t)H * sizeof(float) > 48 * 1024)
     return ULLM_ERR_SHAPE;
-  const size_t lds = (size_t)H * sizeof(float);
-  if (dtype == ULLM_F32)
-    hipLaunchKernelGGL(moe_router_kernel<float>, dim3(T_), dim3(256), lds, stream, (const float*)x, ldx, w, correction, H,
-                       n_router, top, ids, weights);
-  else if (dtype == ULLM_BF16)
-    hipLaunchKernelGGL(moe_router_kernel<bf16_t>, dim3(T_), dim3(256), lds, stream, (const bf16_t*)x, ldx, w, correction, H,
-                       n_router, top, ids, weights);
-  else
-    return ULLM_ERR_DTYPE;
+  // many tokens: four a block, so that a piece of the router's matrix is fetched once for four rows (where their rows
+  // and four sets of scores fit shared memory); few: a block each
+  const bool four = T_ >= 512 && (size_t)H * sizeof(float) <= 8 * 1024 && n_router <= 256;
+  const size_t lds = (size_t)H * sizeof(float) * (four ? 4 : 1);
+  dim3 grid(four ? (T_ + 3) / 4 : T_), block(256);
+#define GO(TT, N) hipLaunchKernelGGL((moe_router_kernel<TT, N>), grid, block, lds, stream, (const TT*)x, ldx, w, correction, T_, H, \
+    n_router, top, ids, weights)
+  if (dtype == ULLM_F32) { if (four) GO(float, 4); else GO(float, 1); }
+  else if (dtype == ULLM_BF16) { if (four) GO(bf16_t, 4); else GO(bf16_t, 1); }
+  else return ULLM_ERR_DTYPE;
+#undef GO
   ULLM_LAUNCH_CHECK();
 }
 
@@ -455,40 +473,35 @@ moe_tiles_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const int* __restri
   }
   const int last_piece = K - 8;
   const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
-  uint4 xreg[2], wreg[4];
-  auto fetch = [&](int k0) __attribute__((always_inline)) {
+  // two sets of registers: a stage is fetched two stages before its products, written to shared memory one before
+  uint4 xreg[2][2], wreg[2][4];
+  auto fetch = [&](int set, int k0) __attribute__((always_inline)) {
     const int k = k0 + 8 * pc;
     const bool in = k <= last_piece;
     const int kk = in ? k : last_piece;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) xreg[i] = ld16(xsrc[i] + kk);
+    for (int i = 0; i < 2; ++i) xreg[set][i] = ld16(xsrc[i] + kk);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) wreg[i] = ld_stream16(wsrc[i] + kk);
+    for (int i = 0; i < 4; ++i) wreg[set][i] = ld_stream16(wsrc[i] + kk);
     if (!in) {
 #pragma unroll
-      for (int i = 0; i < 2; ++i) xreg[i] = zero;
+      for (int i = 0; i < 2; ++i) xreg[set][i] = zero;
     }
+  };
+  auto put = [&](int set, int buf) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) st16(xs2[buf] + xput[i], xreg[set][i]);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) st16(ws2[buf] + wput[i], wreg[set][i]);
   };
   f32x4_t acc[2][4];
 #pragma unroll
   for (int h = 0; h < 2; ++h)
 #pragma unroll
     for (int t = 0; t < 4; ++t) acc[h][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  auto put = [&](int buf) __attribute__((always_inline)) {
-#pragma unroll
-    for (int i = 0; i < 2; ++i) st16(xs2[buf] + xput[i], xreg[i]);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) st16(ws2[buf] + wput[i], wreg[i]);
-  };
-  fetch(0);
-  put(0);
-  __syncthreads();
-  int cur = 0;
-  for (int k0 = 0; k0 < K; k0 += 64, cur ^= 1) {
-    const bool more = k0 + 64 < K;
-    if (more) fetch(k0 + 64);                             // on its way while this stage's products run
-    const unsigned char* xs = xs2[cur];
-    const unsigned char* ws = ws2[cur];
+  auto products = [&](int buf) __attribute__((always_inline)) {
+    const unsigned char* xs = xs2[buf];
+    const unsigned char* ws = ws2[buf];
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
       Pack8 a[2], b[4];
@@ -507,8 +520,22 @@ moe_tiles_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const int* __restri
 #pragma unroll
         for (int t = 0; t < 4; ++t) acc[h][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[h].v, b[t].v, acc[h][t], 0, 0, 0);
     }
-    // the other stage was last read before the barrier that ended the step before: it can be written now
-    if (more) put(cur ^ 1);
+  };
+  fetch(0, 0);
+  put(0, 0);
+  __syncthreads();
+  if (64 < K) fetch(0, 64);
+  for (int k0 = 0; k0 < K; k0 += 128) {
+    // stage k0 lies in buffer 0, set 0 holds stage k0 + 64 (on its way)
+    if (k0 + 128 < K) fetch(1, k0 + 128);
+    products(0);
+    if (k0 + 64 < K) put(0, 1);          // buffer 1 was last read before the barrier that ended the step before
+    __syncthreads();
+    if (k0 + 64 >= K) break;
+    // stage k0 + 64 lies in buffer 1, set 1 holds stage k0 + 128
+    if (k0 + 192 < K) fetch(0, k0 + 192);
+    products(1);
+    if (k0 + 128 < K) put(1, 0);
     __syncthreads();
   }
   // lane (r, g): row r of each 16-row group; columns 16 wave + 4g .. + 4 of the block's (and 64 further on)
