@@ -441,15 +441,22 @@ moe_rows_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const int* __restric
 template <bool GATED>
 __global__ void __launch_bounds__(256)
 moe_tiles_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const int* __restrict__ row_index,
-                      const bf16_t* __restrict__ w, const int* __restrict__ tiles, void* __restrict__ out_, int ldo,
-                      int n_out, int K, float limit, float alpha) {
+                      const bf16_t* __restrict__ w, const int* __restrict__ tiles, int n_tiles, int n_col_blocks,
+                      void* __restrict__ out_, int ldo, int n_out, int K, float limit, float alpha) {
   __shared__ __attribute__((aligned(16))) unsigned char xs2[2][64 * 128];      // two stages take turns
   __shared__ __attribute__((aligned(16))) unsigned char ws2[2][128 * 128];
-  const int tile = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 15, g = lane >> 4;
+  // Workgroups go to the chip's 8 dies round-robin by their id and every die has a second-level cache of its own:
+  // die d takes the d-th eighth of the work (column block by column block, tiles in the list's order), so that the
+  // tiles of one expert, which read the same rows of its matrix, run on one die at about the same time.
+  const int total = n_tiles * n_col_blocks, per_die = (total + 7) / 8;
+  const int item = ((int)blockIdx.x & 7) * per_die + ((int)blockIdx.x >> 3);
+  if ((int)(blockIdx.x >> 3) >= per_die || item >= total) return;
+  const int tile = item % n_tiles, col_block = item / n_tiles;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 15, g = lane >> 4;
   const int e = tiles[3 * tile], slot0 = tiles[3 * tile + 1], rows = tiles[3 * tile + 2];
   if (rows <= 0) return;
   const int cols = GATED ? 64 : 128;                      // output columns of a block
-  const int n0 = blockIdx.y * cols;
+  const int n0 = col_block * cols;
   const size_t w_rows = GATED ? 2 * (size_t)n_out : (size_t)n_out;
   const bf16_t* we = w + (size_t)e * w_rows * K;
   // what this thread fetches of a stage: piece `pc` of x rows prow, prow + 32 and of matrix rows prow + 32 i
@@ -587,14 +594,16 @@ extern "C" int ullm_moe_rows(const void* x, int ldx, const int* row_index, const
   if (n_out < 1 || K < 1 || ldx < K || ldo < n_out || tile_rows < 1) return ULLM_ERR_SHAPE;
   if (dtype == ULLM_BF16 && ullm_moe_mfma_supports(K, ldx, tile_rows) && !((uintptr_t)x & 15) && !((uintptr_t)w & 15)) {
     if (tile_rows == 64) {
-      dim3 grid(max_tiles, (n_out + (gated ? 63 : 127)) / (gated ? 64 : 128)), block(256);
-      if (grid.y > 65535) return ULLM_ERR_SHAPE;
+      const int col_blocks = (n_out + (gated ? 63 : 127)) / (gated ? 64 : 128);
+      const long long total = (long long)max_tiles * col_blocks;
+      if (total > 0x3fffffffLL) return ULLM_ERR_SHAPE;
+      dim3 grid((unsigned)(8 * ((total + 7) / 8))), block(256);
       if (gated)
         hipLaunchKernelGGL(moe_tiles_mfma_kernel<true>, grid, block, 0, stream, (const bf16_t*)x, ldx, row_index,
-                           (const bf16_t*)w, tiles, out, ldo, n_out, K, limit, alpha);
+                           (const bf16_t*)w, tiles, max_tiles, col_blocks, out, ldo, n_out, K, limit, alpha);
       else
         hipLaunchKernelGGL(moe_tiles_mfma_kernel<false>, grid, block, 0, stream, (const bf16_t*)x, ldx, row_index,
-                           (const bf16_t*)w, tiles, out, ldo, n_out, K, limit, alpha);
+                           (const bf16_t*)w, tiles, max_tiles, col_blocks, out, ldo, n_out, K, limit, alpha);
       ULLM_LAUNCH_CHECK();
     }
     dim3 grid(max_tiles, (n_out + 15) / 16), block(256);
