@@ -431,20 +431,23 @@ moe_rows_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const int* __restric
   }
 }
 
-// Many rows a tile (prompt portions): grid (tiles, blocks of 128 rows of the expert's matrix); tile = up to 64 grouped
-// rows of one expert.  A stage is 64 values of K: the tile's 64 rows of x and 128 rows of the matrix (GATED: the
+// Many rows a tile (prompt portions): a block per (tile, 128 rows of the expert's matrix); tile = up to 16 MT = 64 or 128
+// grouped rows of one expert.  A stage is 64 values of K: the tile's rows of x and 128 rows of the matrix (GATED: the
 // gate rows and the up rows of 64 output columns; else 128 output columns) go through shared memory once a block,
 // 128-byte rows whose 16-byte piece c of row r lies at piece c ^ ((r >> 1) & 7) (the 16 lanes the hardware serves
 // together then read 16 different bank groups); the next stage is fetched into registers while the products of this
 // one run.  Wave v takes matrix rows 16 v .. and 64 + 16 v .. (GATED: gate and up of the same columns) against all
-// 64 rows of x: 16 products per 12 reads of shared memory.
-template <bool GATED>
+// rows of x: 16 products per 12 reads of shared memory at 64 rows, 32 per 20 at 128 (and 64 rather than 43 products
+// per byte fetched).
+template <int MT, bool GATED>
 __global__ void __launch_bounds__(256)
 moe_tiles_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const int* __restrict__ row_index,
                       const bf16_t* __restrict__ w, const int* __restrict__ tiles, int n_tiles, int n_col_blocks,
                       void* __restrict__ out_, int ldo, int n_out, int K, float limit, float alpha) {
-  __shared__ __attribute__((aligned(16))) unsigned char xs2[2][64 * 128];      // two stages take turns
-  __shared__ __attribute__((aligned(16))) unsigned char ws2[2][128 * 128];
+  extern __shared__ __attribute__((aligned(16))) unsigned char tile_stages[];  // two stages take turns: x, then the matrix
+  constexpr int XB = 16 * MT * 128, WB = 128 * 128;
+  unsigned char* const xs2[2] = {tile_stages, tile_stages + XB + WB};
+  unsigned char* const ws2[2] = {tile_stages + XB, tile_stages + 2 * XB + WB};
   // Workgroups go to the chip's 8 dies round-robin by their id and every die has a second-level cache of its own:
   // die d takes the d-th eighth of the work (column block by column block, tiles in the list's order), so that the
   // tiles of one expert, which read the same rows of its matrix, run on one die at about the same time.
@@ -459,13 +462,14 @@ moe_tiles_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const int* __restri
   const int n0 = col_block * cols;
   const size_t w_rows = GATED ? 2 * (size_t)n_out : (size_t)n_out;
   const bf16_t* we = w + (size_t)e * w_rows * K;
-  // what this thread fetches of a stage: piece `pc` of x rows prow, prow + 32 and of matrix rows prow + 32 i
+  // what this thread fetches of a stage: piece `pc` of x rows prow + 32 i and of matrix rows prow + 32 i
+  constexpr int XP = MT / 2;                              // pieces of x a thread fetches a stage
   const int pc = tid & 7, prow = tid >> 3;
-  const bf16_t* xsrc[2];
+  const bf16_t* xsrc[XP];
   const bf16_t* wsrc[4];
-  int xput[2], wput[4];
+  int xput[XP], wput[4];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
+  for (int i = 0; i < XP; ++i) {
     const int row = prow + 32 * i, rr = row < rows ? row : rows - 1;
     xsrc[i] = x + (size_t)(row_index ? row_index[slot0 + rr] : slot0 + rr) * ldx;
     xput[i] = row * 128 + ((pc ^ ((row >> 1) & 7)) << 4);
@@ -481,52 +485,56 @@ moe_tiles_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const int* __restri
   const int last_piece = K - 8;
   const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
   // two sets of registers: a stage is fetched two stages before its products, written to shared memory one before
-  uint4 xreg[2][2], wreg[2][4];
+  uint4 xreg[2][XP], wreg[2][4];
   auto fetch = [&](int set, int k0) __attribute__((always_inline)) {
     const int k = k0 + 8 * pc;
     const bool in = k <= last_piece;
     const int kk = in ? k : last_piece;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) xreg[set][i] = ld16(xsrc[i] + kk);
+    for (int i = 0; i < XP; ++i) xreg[set][i] = ld16(xsrc[i] + kk);
 #pragma unroll
     for (int i = 0; i < 4; ++i) wreg[set][i] = ld_stream16(wsrc[i] + kk);
     if (!in) {
 #pragma unroll
-      for (int i = 0; i < 2; ++i) xreg[set][i] = zero;
+      for (int i = 0; i < XP; ++i) xreg[set][i] = zero;
     }
   };
   auto put = [&](int set, int buf) __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) st16(xs2[buf] + xput[i], xreg[set][i]);
+    for (int i = 0; i < XP; ++i) st16(xs2[buf] + xput[i], xreg[set][i]);
 #pragma unroll
     for (int i = 0; i < 4; ++i) st16(ws2[buf] + wput[i], wreg[set][i]);
   };
-  f32x4_t acc[2][4];
+  f32x4_t acc[2][MT];
 #pragma unroll
   for (int h = 0; h < 2; ++h)
 #pragma unroll
-    for (int t = 0; t < 4; ++t) acc[h][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t < MT; ++t) acc[h][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   auto products = [&](int buf) __attribute__((always_inline)) {
     const unsigned char* xs = xs2[buf];
     const unsigned char* ws = ws2[buf];
+    // both steps of 32 are read before the first product: the second step's reads travel during the first's products
+    Pack8 a[2][2], b[2][MT];
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
-      Pack8 a[2], b[4];
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
         const int row = 64 * h + 16 * wave + r;
-        a[h].u4 = ld16(ws + row * 128 + (((4 * s + g) ^ ((row >> 1) & 7)) << 4));
+        a[s][h].u4 = ld16(ws + row * 128 + (((4 * s + g) ^ ((row >> 1) & 7)) << 4));
       }
 #pragma unroll
-      for (int t = 0; t < 4; ++t) {
+      for (int t = 0; t < MT; ++t) {
         const int row = 16 * t + r;
-        b[t].u4 = ld16(xs + row * 128 + (((4 * s + g) ^ ((row >> 1) & 7)) << 4));
+        b[s][t].u4 = ld16(xs + row * 128 + (((4 * s + g) ^ ((row >> 1) & 7)) << 4));
       }
+    }
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
 #pragma unroll
       for (int h = 0; h < 2; ++h)
 #pragma unroll
-        for (int t = 0; t < 4; ++t) acc[h][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[h].v, b[t].v, acc[h][t], 0, 0, 0);
-    }
+        for (int t = 0; t < MT; ++t)
+          acc[h][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[s][h].v, b[s][t].v, acc[h][t], 0, 0, 0);
   };
   fetch(0, 0);
   put(0, 0);
@@ -547,7 +555,7 @@ moe_tiles_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const int* __restri
   }
   // lane (r, g): row r of each 16-row group; columns 16 wave + 4g .. + 4 of the block's (and 64 further on)
 #pragma unroll
-  for (int t = 0; t < 4; ++t) {
+  for (int t = 0; t < MT; ++t) {
     const int row = 16 * t + r;
     if (row >= rows) continue;
     if (GATED) {
@@ -582,7 +590,16 @@ moe_tiles_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const int* __restri
 
 // Rows of a tile the matrix-core kernels take for a launch made with `tile_rows` rows a tile.
 extern "C" int ullm_moe_mfma_supports(int K, int ldx, int tile_rows) {
-  return K >= 8 && K % 8 == 0 && ldx % 8 == 0 && (tile_rows == 16 || tile_rows == 32 || tile_rows == 64);
+  return K >= 8 && K % 8 == 0 && ldx % 8 == 0 && (tile_rows == 16 || tile_rows == 32 || tile_rows == 64 || tile_rows == 128);
+}
+
+template <int MT, bool GATED, typename... Args>
+static void launch_tiles(dim3 grid, hipStream_t stream, Args... args) {
+  constexpr int bytes = 2 * (16 * MT * 128 + 128 * 128);
+  static const hipError_t allowed = hipFuncSetAttribute((const void*)moe_tiles_mfma_kernel<MT, GATED>,
+                                                        hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  (void)allowed;
+  hipLaunchKernelGGL((moe_tiles_mfma_kernel<MT, GATED>), grid, dim3(256), bytes, stream, args...);
 }
 
 // out[slot] = glu(x[row_index[slot]] Wg^T, x Wu^T) (gated: out in x's dtype, w [experts, 2 n_out, K]) or
@@ -593,17 +610,16 @@ extern "C" int ullm_moe_rows(const void* x, int ldx, const int* row_index, const
   if (max_tiles <= 0) return 0;
   if (n_out < 1 || K < 1 || ldx < K || ldo < n_out || tile_rows < 1) return ULLM_ERR_SHAPE;
   if (dtype == ULLM_BF16 && ullm_moe_mfma_supports(K, ldx, tile_rows) && !((uintptr_t)x & 15) && !((uintptr_t)w & 15)) {
-    if (tile_rows == 64) {
+    if (tile_rows >= 64) {
       const int col_blocks = (n_out + (gated ? 63 : 127)) / (gated ? 64 : 128);
       const long long total = (long long)max_tiles * col_blocks;
       if (total > 0x3fffffffLL) return ULLM_ERR_SHAPE;
-      dim3 grid((unsigned)(8 * ((total + 7) / 8))), block(256);
-      if (gated)
-        hipLaunchKernelGGL(moe_tiles_mfma_kernel<true>, grid, block, 0, stream, (const bf16_t*)x, ldx, row_index,
-                           (const bf16_t*)w, tiles, max_tiles, col_blocks, out, ldo, n_out, K, limit, alpha);
-      else
-        hipLaunchKernelGGL(moe_tiles_mfma_kernel<false>, grid, block, 0, stream, (const bf16_t*)x, ldx, row_index,
-                           (const bf16_t*)w, tiles, max_tiles, col_blocks, out, ldo, n_out, K, limit, alpha);
+      dim3 grid((unsigned)(8 * ((total + 7) / 8)));
+#define TILES(MT, G) launch_tiles<MT, G>(grid, stream, (const bf16_t*)x, ldx, row_index, (const bf16_t*)w, tiles, max_tiles, \
+    col_blocks, out, ldo, n_out, K, limit, alpha)
+      if (tile_rows == 64) { if (gated) TILES(4, true); else TILES(4, false); }
+      else { if (gated) TILES(8, true); else TILES(8, false); }
+#undef TILES
       ULLM_LAUNCH_CHECK();
     }
     dim3 grid(max_tiles, (n_out + 15) / 16), block(256);

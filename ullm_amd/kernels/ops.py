@@ -1050,7 +1050,7 @@ def paged_attention(q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
 # ---------------------------------------------------------------------------------- routed feed-forward
 
 MOE_MAX_ROUTER, MOE_MAX_TOP = 1024, 32
-MOE_TILE_ROWS = (16, 32, 64)     # grouped rows a block of the matrix-core expert products takes
+MOE_TILE_ROWS = (16, 32, 64, 128)     # grouped rows a block of the matrix-core expert products takes
 
 
 def moe_route(logits: torch.Tensor, correction: Optional[torch.Tensor], top: int):

@@ -33,6 +33,8 @@ def tile_rows_for(tokens: int, top: int, experts: int) -> int:
     """Grouped rows a block of the expert products takes, from the rows an expert gets on average: a function of
     the step's size alone."""
     mean = tokens * top / max(1, experts)
+    if mean >= 96:
+        return 128
     if mean >= 48:
         return 64
     return 32 if mean >= 24 else 16
