@@ -111,10 +111,10 @@ extern "C" int ullm_moe_route(const float* logits, int ld, const float* correcti
 // The router's product and the routing in one kernel: a block takes TPB tokens; their rows lie in shared memory as
 // 32-bit values, every wave takes four router outputs at a time with four 16-byte pieces of each of their rows a
 // lane under way (the loop is a chain of trips to memory otherwise), and every piece fetched serves all the block's
-// tokens.  A lane adds a token's pieces in rising order, then the wave adds up: an order that depends on nothing but
+// tokens (four tokens and four waves a block for many tokens; one token and sixteen waves for few).  A lane adds a token's pieces in rising order, then the wave adds up: an order that depends on nothing but
 // the row.  Then wave v routes token v.  The router's matrix is 32-bit [n_router, H].
 template <typename T, int TPB>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(TPB == 1 ? 1024 : 256)
 moe_router_kernel(const T* __restrict__ x, int ldx, const float* __restrict__ w, const float* __restrict__ correction,
                   int n_tokens, int H, int n_router, int top, int* __restrict__ ids, float* __restrict__ weights) {
   extern __shared__ __attribute__((aligned(16))) float xrow[];          // [TPB][H]
@@ -125,11 +125,11 @@ moe_router_kernel(const T* __restrict__ x, int ldx, const float* __restrict__ w,
 #pragma unroll
   for (int q = 0; q < TPB; ++q) {
     const T* xr = x + (size_t)(t0 + q < n_tokens ? t0 + q : n_tokens - 1) * ldx;
-    for (int i = tid; i < H; i += 256) xrow[q * H + i] = ld_f32(xr + i);
+    for (int i = tid; i < H; i += (int)blockDim.x) xrow[q * H + i] = ld_f32(xr + i);
   }
   __syncthreads();
   const bool vec = (H & 3) == 0 && (((uintptr_t)w) & 15) == 0;
-  for (int e0 = 4 * wave; e0 < n_router; e0 += 16) {
+  for (int e0 = 4 * wave; e0 < n_router; e0 += (int)(blockDim.x >> 4)) {
     float a[TPB][4];
 #pragma unroll
     for (int q = 0; q < TPB; ++q)
@@ -192,7 +192,8 @@ extern "C" int ullm_moe_router(const void* x, int ldx, const float* w, const flo
   // and four sets of scores fit shared memory); few: a block each
   const bool four = T_ >= 512 && (size_t)H * sizeof(float) <= 8 * 1024 && n_router <= 256;
   const size_t lds = (size_t)H * sizeof(float) * (four ? 4 : 1);
-  dim3 grid(four ? (T_ + 3) / 4 : T_), block(256);
+  // a token a block: sixteen waves, so that up to 64 router outputs are summed in one round of trips to memory
+  dim3 grid(four ? (T_ + 3) / 4 : T_), block(four ? 256 : 1024);
 #define GO(TT, N) hipLaunchKernelGGL((moe_router_kernel<TT, N>), grid, block, lds, stream, (const TT*)x, ldx, w, correction, T_, H, \
     n_router, top, ids, weights)
   if (dtype == ULLM_F32) { if (four) GO(float, 4); else GO(float, 1); }
