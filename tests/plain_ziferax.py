@@ -78,10 +78,17 @@ def expert(w, prefix: str, limit: float, h: torch.Tensor) -> torch.Tensor:
     return clamped_unit(h @ w[f"{prefix}.gate"].T, h @ w[f"{prefix}.up"].T, limit) @ w[f"{prefix}.down"].T
 
 
+MARGINS = None      # a list: route() then appends, per call, every token's gap between the last choice score taken and the first left
+
+
 def route(w, prefix: str, r: dict, h: torch.Tensor):
     """(indices [T, top], weights [T, top]): softmax over all router outputs, the choice by score + correction,
     the weights by the chosen scores over their sum."""
     s = torch.softmax(h @ w[f"{prefix}.router"].T, -1)
+    if MARGINS is not None:
+        ranked = torch.sort(s + w[f"{prefix}.correction"], dim=-1, descending=True).values
+        MARGINS.append(ranked[:, r["top"] - 1] - ranked[:, r["top"]] if r["top"] < ranked.shape[1]
+                       else torch.full((h.shape[0],), math.inf, dtype=h.dtype))
     chosen = torch.topk(s + w[f"{prefix}.correction"], r["top"], dim=-1).indices
     picked = torch.gather(s, 1, chosen)
     return chosen, picked / (picked.sum(-1, keepdim=True) + 1e-20)
@@ -133,11 +140,15 @@ def greedy_generate(w, cfg, prompt: List[int], n: int) -> List[int]:
 
 
 def random_weights(cfg: dict, seed: int, std: float = 0.08, sink_std: float = 1.0, correction_std: float = 0.05,
-                   router_std: float = 0.5) -> Dict[str, torch.Tensor]:
+                   router_std: Optional[float] = None) -> Dict[str, torch.Tensor]:
     """bfloat16 tensors under the design's names.  Sinks of about one unit and a router whose scores differ: a sink
-    left out, or a correction that leaks into the weights, then moves the logits far beyond rounding."""
+    left out, or a correction that leaks into the weights, then moves the logits far beyond rounding.  The router's
+    logits are about a unit and a half wide whatever the width (a saturated softmax leaves the choice among the
+    others to the corrections, whose bfloat16 values tie)."""
     g = torch.Generator().manual_seed(seed)
     H = cfg["width"]
+    if router_std is None:
+        router_std = 1.5 / math.sqrt(H)
 
     def mat(*shape, s=std):
         return (torch.randn(*shape, generator=g) * s).bfloat16()

@@ -21,9 +21,9 @@ pytestmark = pytest.mark.gpu
 
 def drawn_layer(rng):
     kv = rng.choice([1, 1, 2, 3, 4])
-    dim = rng.choice([8, 16, 24, 32, 40, 48, 64, 80, 96, 128])
+    dim = rng.choice([8, 12, 16, 20, 24, 32, 40, 48, 64, 72, 80, 96, 128, 160, 256, 288])
     rot = rng.choice([0, 2, dim // 2 - (dim // 2) % 2, dim])
-    mixer = dict(heads=kv * rng.choice([1, 2, 3, 4, 8]), kv_heads=kv, dim=dim, vdim=dim,
+    mixer = dict(heads=kv * rng.choice([1, 2, 3, 4, 8, 20]), kv_heads=kv, dim=dim, vdim=dim,
                  mask=dict(size=rng.choice([1, 2, 5, 15, 16, 17, 31, 32, 33, 48, 64, 100, 500])),
                  rot=dict(base=rng.choice([100.0, 10000.0, 500000.0]), dims=rot), scale=rng.choice([0.05, 0.125, 0.3]))
     if rot == 0:
@@ -32,7 +32,7 @@ def drawn_layer(rng):
     if rng.random() < 0.8:
         experts, identity = rng.choice([1, 2, 3, 5, 8, 16, 40]), rng.choice([0, 0, 1, 2, 5])
         mlp = dict(kind="moe", router=dict(experts=experts, identity=identity, top=rng.randint(1, min(6, experts + identity))),
-                   expert=dict(ff=rng.choice([4, 8, 12, 16, 24, 40, 64, 100]), limit=rng.choice([0.5, 1.5, 7.0])))
+                   expert=dict(ff=rng.choice([4, 6, 8, 12, 16, 24, 40, 64, 100, 130]), limit=rng.choice([0.5, 1.5, 7.0])))
         if rng.random() < 0.6:
             mlp["shared"] = dict(ff=rng.choice([8, 20, 64, 136]), limit=rng.choice([0.5, 2.0]))
     return dict(type="attention", mixer=mixer, mlp=mlp)
@@ -47,12 +47,12 @@ def drawn_config(rng):
             layers.append(dict(json.loads(json.dumps(layers[src])), weights_of=src))
         else:
             layers.append(drawn_layer(rng))
-    return dict(architecture="Ziferax", vocab=rng.randint(40, 700), width=rng.choice([24, 32, 40, 48, 64, 72, 96, 128, 160, 256]),
+    return dict(architecture="Ziferax", vocab=rng.randint(40, 700), width=rng.choice([20, 24, 32, 36, 40, 48, 50, 64, 72, 96, 100, 128, 160, 256]),
                 layers=layers, norm=dict(eps=rng.choice([1e-5, 1e-6, 1e-3])), residual_mult=rng.choice([0.3, 0.5, 1.0, 0.7]))
 
 
 def worst_error(got, want):
-    return float(np.abs(got - want).max() / np.abs(want).max())
+    return float(np.abs(got - want).max() / np.abs(want).max()) if len(want) else 0.0
 
 
 def schedules(rep, rng, reqs):
@@ -105,16 +105,29 @@ def test_drawn_configurations(seed, tmp_path):
     save_file({k: v.contiguous() for k, v in w.items()}, os.path.join(tmp_path, "model.safetensors"))
     wide = {k: v.double() for k, v in w.items()}
     reqs = {f"r{i}": [rng.randrange(cfg["vocab"]) for _ in range(rng.randint(20, 110))] for i in range(6)}
-    want = {k: plain.forward(wide, cfg, t).float().numpy() for k, t in reqs.items()}
+    want, sharp = {}, {}
+    for k, t in reqs.items():
+        plain.MARGINS = []
+        want[k] = plain.forward(wide, cfg, t).float().numpy()
+        # rows before the first token whose router nearly ties (32-bit sums may settle it otherwise, and every later
+        # row may see that token): only these are held to the 32-bit bound
+        gaps = np.min([m.numpy() for m in plain.MARGINS], axis=0) if plain.MARGINS else np.full(len(t), np.inf)
+        plain.MARGINS = None
+        close_calls = np.nonzero(gaps < 1e-5)[0]
+        sharp[k] = int(close_calls[0]) if len(close_calls) else len(t)
+    assert sum(sharp.values()) >= 0.5 * sum(len(t) for t in reqs.values()), ("near-ties leave too few rows to compare", sharp)
     narrow = {k: v.float() for k, v in w.items()}
     # what 32-bit sums alone do to this model (four times that, as the engine sums in another order), at least 3e-5
-    bound = {k: max(3e-5, 4 * worst_error(plain.forward(narrow, cfg, t).numpy(), want[k])) for k, t in reqs.items()}
+    bound = {k: max(3e-5, 4 * worst_error(plain.forward(narrow, cfg, t).numpy()[:sharp[k]], want[k][:sharp[k]])) if sharp[k] else 1.0
+             for k, t in reqs.items()}
     state = rng.getstate()
     whole, cut, mixed = schedules(Replayer(str(tmp_path), "float32", 512, 16, DEV, max_requests=4), rng, reqs)
-    assert worst_error(whole, want["r0"]) <= bound["r0"] and worst_error(cut, want["r0"]) <= bound["r0"]
-    assert np.array_equal(whole, cut)                       # 32-bit sums are ordered by the row alone
+    n0 = sharp["r0"]
+    assert worst_error(whole[:n0], want["r0"][:n0]) <= bound["r0"], ("whole", worst_error(whole[:n0], want["r0"][:n0]), bound["r0"])
+    assert worst_error(cut[:n0], want["r0"][:n0]) <= bound["r0"], ("cut", worst_error(cut[:n0], want["r0"][:n0]), bound["r0"])
+    assert np.array_equal(whole, cut), "whole and cut differ in 32-bit"      # 32-bit sums are ordered by the row alone
     for k in reqs:
-        assert worst_error(mixed[k], want[k]) <= bound[k], k
+        assert worst_error(mixed[k][:sharp[k]], want[k][:sharp[k]]) <= bound[k], k
     # bfloat16: the same schedules.  What rounding does to a routed model depends on the model (a rounded router input
     # picks another expert at a close call, and then a whole row moves), so the bounds are multiples of what the plain
     # implementation loses when nothing but its sublayers' inputs are rounded to bfloat16: for the middle row and for
@@ -124,9 +137,8 @@ def test_drawn_configurations(seed, tmp_path):
     whole, cut, mixed = schedules(rep, rng, reqs)
     alone = {k: rep.step({"step": 0, "entries": [{"id": "a", "tokens": t, "want": list(range(len(t)))}], "end": ["a"]})
              for k, t in reqs.items()}
-    floor = np.concatenate([np.abs(plain.forward(wide, cfg, t, round_to=torch.bfloat16).float().numpy() - want[k]).max(-1)
-                            / np.abs(want[k]).max() for k, t in reqs.items()])
-    mid, most = 5e-3 + 4 * float(np.median(floor)), 1e-2 + 4 * float(np.quantile(floor, 0.85))
-    for got, ref in [(whole, want["r0"]), (cut, whole)] + [(mixed[k], alone[k]) for k in reqs]:
+    for got, ref, k in [(whole, want["r0"], "r0"), (cut, whole, "r0")] + [(mixed[k], alone[k], k) for k in reqs]:
+        floor = np.abs(plain.forward(wide, cfg, reqs[k], round_to=torch.bfloat16).float().numpy() - want[k]).max(-1) / np.abs(want[k]).max()
+        mid, most = 5e-3 + 4 * float(np.median(floor)), 1e-2 + 4 * float(np.quantile(floor, 0.85))
         err = np.abs(got - ref).max(-1) / np.abs(ref).max()
-        assert np.median(err) <= mid and np.quantile(err, 0.85) <= most, (float(np.median(err)), float(np.quantile(err, 0.85)), mid, most)
+        assert np.median(err) <= mid and np.quantile(err, 0.85) <= most, (k, float(np.median(err)), float(np.quantile(err, 0.85)), mid, most)

@@ -49,6 +49,7 @@ def test_a_layer_that_uses_another_layers_tensors_declares_none_and_keeps_a_cach
     (lambda c: c["layers"][0]["mlp"]["router"].update(top=9), "top"),
     (lambda c: c["layers"][0]["mlp"].update(kind="dense"), "kind"),
     (lambda c: c["layers"][2].update(weights_of=2), "weights_of"),
+    (lambda c: c["layers"][2].update(weights_of=7), "weights_of"),
     (lambda c: c["layers"][2].update(weights_of=1), "differ"),
     (lambda c: c["layers"][1].update(type="mamba2"), "type"),
     (lambda c: c.pop("width"), "width"),
@@ -68,3 +69,11 @@ def test_keys_a_model_may_leave_out():
     c.pop("residual_mult")
     cfg = ZiferaxConfig.from_dict(c)
     assert cfg.layers[0].mlp.shared_ff == 0 and cfg.layers[0].mlp.identity == 0 and cfg.residual_mult == 1.0
+
+
+def test_a_chain_of_layers_that_use_anothers_tensors_is_followed():
+    c = base()
+    c["layers"].append(dict(copy.deepcopy(c["layers"][0]), weights_of=2))
+    cfg = ZiferaxConfig.from_dict(c)
+    assert cfg.layers[3].weights_of == 0
+    assert build_model(c)[1].run_order == [(0, 0), (1, 1), (0, 2), (0, 3)]

@@ -390,8 +390,14 @@ class ZiferaxConfig:
                 src = L.get("weights_of")
                 if src is not None:
                     src = _take(L, "weights_of", int)
-                    if not 0 <= src < len(raw_layers) or src == i or raw_layers[src].get("weights_of") is not None:
-                        raise ConfigError(f"'weights_of': {src} must name another layer with tensors of its own")
+                    seen = {i}
+                    while True:                                   # a layer may name one that names another: followed to the tensors
+                        if not 0 <= src < len(raw_layers) or src in seen or not isinstance(raw_layers[src], Mapping):
+                            raise ConfigError(f"'weights_of': {src} must lead to another layer with tensors of its own")
+                        if raw_layers[src].get("weights_of") is None:
+                            break
+                        seen.add(src)
+                        src = _take(raw_layers[src], "weights_of", int)
             except ConfigError as e:
                 raise ConfigError(f"{e} (layer {i})") from None
             layers.append(ZiferaxLayer(kind, att, mlp, src))
