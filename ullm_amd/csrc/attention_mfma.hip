@@ -1398,9 +1398,11 @@ attention_prefill_dma_kernel(const bf16_t* __restrict__ q, int q_stride, bf16_t*
   using BiasPtr = typename BiasPointer<EXTRA>::type;
   BiasPtr bias_row = nullptr;
   if constexpr (EXTRA) {
-    const float* const bias_global = extras.bias + (size_t)head * extras.bias_rows;
-    for (int i = lane + 64 * half; i <= bias_last; i += 64 * KS) dma_bias_stage[wave * extras.bias_rows + i] = bias_global[i];
-    bias_row = (lds_bias_ptr)dma_bias_stage + wave * extras.bias_rows;
+    if (extras.bias) {                                    // extras without a bias (a gate, a sink) stage nothing
+      const float* const bias_global = extras.bias + (size_t)head * extras.bias_rows;
+      for (int i = lane + 64 * half; i <= bias_last; i += 64 * KS) dma_bias_stage[wave * extras.bias_rows + i] = bias_global[i];
+      bias_row = (lds_bias_ptr)dma_bias_stage + wave * extras.bias_rows;
+    }
   }
   const int first = tiles[2 * tile_idx], count = tiles[2 * tile_idx + 1];
   int clo[NG], chi[NG], tok[NG];
@@ -1750,9 +1752,9 @@ extern "C" int ullm_attention_decode_static(
 #define BIAS_STAGE_MAX (PREFILL_WAVES * BIAS_STAGE_ROWS * (int)sizeof(float))
 #define DMA_BIAS_ROWS 1792                // what fits beside four tiles a half and the page ids, for both halves
 template <int N, typename... Args>
-static void prefill_launch_extras(int halves, size_t bias_bytes, unsigned blocks, hipStream_t stream, Args... args) {
+static void prefill_launch_extras(int halves, size_t bias_bytes, bool no_bias, unsigned blocks, hipStream_t stream, Args... args) {
   if constexpr (N == 4) {                 // tiles straight to shared memory, as without extras
-    if (bias_bytes && bias_bytes <= (size_t)PREFILL_WAVES * DMA_BIAS_ROWS * sizeof(float)) {
+    if (no_bias || (bias_bytes && bias_bytes <= (size_t)PREFILL_WAVES * DMA_BIAS_ROWS * sizeof(float))) {
       if (halves == 2) {
         static const hipError_t allowed = hipFuncSetAttribute((const void*)attention_prefill_dma_kernel<N, 2, true>,
             hipFuncAttributeMaxDynamicSharedMemorySize, PREFILL_WAVES * DMA_BIAS_ROWS * (int)sizeof(float));
@@ -1868,7 +1870,7 @@ static int prefill_any(
   // rows of up to 2048 distances go to shared memory (four heads a block: 32 KiB at most beside the tiles)
   const size_t bias_bytes = extras && extras->bias && extras->bias_rows <= BIAS_STAGE_ROWS
                                 ? (size_t)PREFILL_WAVES * extras->bias_rows * sizeof(float) : 0;
-#define CALL_EXTRA(N) prefill_launch_extras<N>(halves, bias_bytes, (unsigned)blocks, stream, (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, \
+#define CALL_EXTRA(N) prefill_launch_extras<N>(halves, bias_bytes, extras->bias == nullptr, (unsigned)blocks, stream, (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, \
     (const bf16_t*)k_pool, (const bf16_t*)v_pool, tiles, positions, token_entry, block_table, bt_stride, page_size,    \
     nq, nkv, sl, window, n_tiles, *extras)
   if (extras) {
