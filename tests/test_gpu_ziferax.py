@@ -470,8 +470,9 @@ def test_grouping_pairs_by_expert(T, top, E, extra, rows):
     for p in torch.nonzero(real).view(-1).tolist():
         e, s = int(flat[p]), int(slot[p])
         assert offsets[e] <= s < offsets[e + 1] and int(token[s]) == p // top
+    assert tiles[-1].tolist() == [int((tiles[:-1, 2] > 0).sum()), 0, 0]          # behind the list: the tiles in use
     covered = []
-    for e, first, n in tiles.tolist():
+    for e, first, n in tiles[:-1].tolist():
         assert 0 <= n <= rows
         if n:
             assert offsets[e] <= first and first + n <= offsets[e + 1]

@@ -205,7 +205,8 @@ extern "C" int ullm_moe_router(const void* x, int ldx, const float* w, const flo
 
 // ------------------------------------------------------------------------------- grouping by expert
 // One block.  offsets [experts + 1]; slot_of_pair [pairs] (-1: the pair's expert has no weights); token_of_slot [pairs];
-// tiles [max_tiles][3] = (expert, first slot, rows), rows 0 for the tiles no expert filled.
+// tiles [max_tiles + 1][3] = (expert, first slot, rows), rows 0 for the tiles no expert filled; the entry behind the
+// list holds the number of tiles in use.
 __global__ void __launch_bounds__(1024)
 moe_sort_kernel(const int* __restrict__ ids, int n_pairs, int top, int n_experts, int tile_rows,
                 int* __restrict__ offsets, int* __restrict__ slot_of_pair, int* __restrict__ token_of_slot,
@@ -255,6 +256,11 @@ moe_sort_kernel(const int* __restrict__ ids, int n_pairs, int top, int n_experts
     tiles[3 * i] = 0;
     tiles[3 * i + 1] = 0;
     tiles[3 * i + 2] = 0;
+  }
+  if (tid == 0) {                                         // one more entry behind the list: how many tiles are in use
+    tiles[3 * max_tiles] = tile_base[n_experts] < max_tiles ? tile_base[n_experts] : max_tiles;
+    tiles[3 * max_tiles + 1] = 0;
+    tiles[3 * max_tiles + 2] = 0;
   }
 }
 
@@ -450,12 +456,14 @@ moe_tiles_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const int* __restri
   unsigned char* const xs2[2] = {tile_stages, tile_stages + XB + WB};
   unsigned char* const ws2[2] = {tile_stages + XB, tile_stages + 2 * XB + WB};
   // Workgroups go to the chip's 8 dies round-robin by their id and every die has a second-level cache of its own:
-  // die d takes the d-th eighth of the work (column block by column block, tiles in the list's order), so that the
-  // tiles of one expert, which read the same rows of its matrix, run on one die at about the same time.
-  const int total = n_tiles * n_col_blocks, per_die = (total + 7) / 8;
+  // die d takes the d-th eighth of the tiles in use, tile by tile in the list's order with all of a tile's column
+  // blocks side by side.  What runs on a die at one time is then a few tiles of one or two experts: a tile's rows
+  // of x are fetched once for all its column blocks, an expert's matrix once for all its tiles.
+  const int used = tiles[3 * n_tiles];
+  const int total = used * n_col_blocks, per_die = (total + 7) / 8;
   const int item = ((int)blockIdx.x & 7) * per_die + ((int)blockIdx.x >> 3);
   if ((int)(blockIdx.x >> 3) >= per_die || item >= total) return;
-  const int tile = item % n_tiles, col_block = item / n_tiles;
+  const int tile = item / n_col_blocks, col_block = item % n_col_blocks;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 15, g = lane >> 4;
   const int e = tiles[3 * tile], slot0 = tiles[3 * tile + 1], rows = tiles[3 * tile + 2];
   if (rows <= 0) return;
@@ -494,7 +502,7 @@ moe_tiles_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const int* __restri
 #pragma unroll
     for (int i = 0; i < XP; ++i) xreg[set][i] = ld16(xsrc[i] + kk);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) wreg[set][i] = ld_stream16(wsrc[i] + kk);
+    for (int i = 0; i < 4; ++i) wreg[set][i] = ld16(wsrc[i] + kk);    // the expert's other tiles read the same rows: cached
     if (!in) {
 #pragma unroll
       for (int i = 0; i < XP; ++i) xreg[set][i] = zero;
@@ -537,19 +545,21 @@ moe_tiles_mfma_kernel(const bf16_t* __restrict__ x, int ldx, const int* __restri
         for (int t = 0; t < MT; ++t)
           acc[h][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[s][h].v, b[s][t].v, acc[h][t], 0, 0, 0);
   };
+  // No fetch stands under a condition (the compiler then waits for every load under way at the next use of any): a
+  // stage past the end of K reads the rows' last pieces again and is never written to shared memory.
   fetch(0, 0);
   put(0, 0);
   __syncthreads();
-  if (64 < K) fetch(0, 64);
+  fetch(0, 64);
   for (int k0 = 0; k0 < K; k0 += 128) {
     // stage k0 lies in buffer 0, set 0 holds stage k0 + 64 (on its way)
-    if (k0 + 128 < K) fetch(1, k0 + 128);
+    fetch(1, k0 + 128);
     products(0);
     if (k0 + 64 < K) put(0, 1);          // buffer 1 was last read before the barrier that ended the step before
     __syncthreads();
     if (k0 + 64 >= K) break;
     // stage k0 + 64 lies in buffer 1, set 1 holds stage k0 + 128
-    if (k0 + 192 < K) fetch(0, k0 + 192);
+    fetch(0, k0 + 192);
     products(1);
     if (k0 + 128 < K) put(1, 0);
     __syncthreads();

@@ -1102,8 +1102,9 @@ def moe_max_tiles(n_pairs: int, n_experts: int, tile_rows: int) -> int:
 
 def moe_sort(ids: torch.Tensor, n_experts: int, tile_rows: int):
     """Groups the pairs (token, k) of ``ids`` int32 [T, top] by expert.  Returns (slot_of_pair int32 [T * top], -1 for
-    a pair whose expert index is >= ``n_experts``; token_of_slot int32 [T * top]; tiles int32 [max_tiles, 3] =
-    (expert, first slot, rows <= tile_rows), rows 0 in unused tiles; offsets int32 [n_experts + 1])."""
+    a pair whose expert index is >= ``n_experts``; token_of_slot int32 [T * top]; tiles int32 [max_tiles + 1, 3] =
+    (expert, first slot, rows <= tile_rows), rows 0 in unused tiles, and behind the list one entry whose first number
+    counts the tiles in use; offsets int32 [n_experts + 1])."""
     _i32(ids, "ids")
     T, top = ids.shape
     n_pairs = T * top
@@ -1111,7 +1112,7 @@ def moe_sort(ids: torch.Tensor, n_experts: int, tile_rows: int):
     max_tiles = moe_max_tiles(n_pairs, n_experts, tile_rows)
     slot_of_pair = torch.empty(n_pairs, dtype=torch.int32, device=dev)
     token_of_slot = torch.empty(n_pairs, dtype=torch.int32, device=dev)
-    tiles = torch.empty((max_tiles, 3), dtype=torch.int32, device=dev)
+    tiles = torch.empty((max_tiles + 1, 3), dtype=torch.int32, device=dev)     # behind the list: the tiles in use
     offsets = torch.empty(n_experts + 1, dtype=torch.int32, device=dev)
     _check(build.load("moe").ullm_moe_sort(_p(ids), _c_int(n_pairs), _c_int(top), _c_int(n_experts), _c_int(tile_rows),
                                            _p(offsets), _p(slot_of_pair), _p(token_of_slot), _p(tiles), _c_int(max_tiles),
@@ -1137,8 +1138,9 @@ def moe_rows(x: torch.Tensor, row_index: Optional[torch.Tensor], w: torch.Tensor
     else:
         _need(x.shape[0] >= n_slots, "fewer rows than slots")
     out = torch.empty((n_slots, n_out), dtype=x.dtype if gated else torch.float32, device=x.device)
+    _need(tiles.shape[0] >= 2, "the tile list ends with the entry that counts the tiles in use")
     _check(build.load("moe").ullm_moe_rows(_p(x), _c_int(x.stride(0)), _p(row_index), _p(w), _p(tiles),
-                                           _c_int(tiles.shape[0]), _c_int(tile_rows), _p(out), _c_int(out.stride(0)),
+                                           _c_int(tiles.shape[0] - 1), _c_int(tile_rows), _p(out), _c_int(out.stride(0)),
                                            _c_int(n_out), _c_int(K), _c_int(1 if gated else 0), _c_float(limit),
                                            _c_float(alpha), _c_int(_dt(x)), _stream()), "moe_rows")
     return out
