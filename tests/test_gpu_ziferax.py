@@ -483,7 +483,8 @@ def test_grouping_pairs_by_expert(T, top, E, extra, rows):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("T,top,E,H,ff,rows", [(5, 2, 4, 64, 32, 16), (70, 3, 5, 136, 72, 16), (200, 2, 3, 128, 64, 64),
                                                (90, 4, 6, 96, 40, 32), (9, 2, 3, 40, 12, 16), (3, 1, 2, 72, 8, 16),
-                                               (300, 3, 4, 200, 136, 64), (130, 2, 2, 72, 200, 64), (500, 3, 4, 264, 72, 128)])
+                                               (300, 3, 4, 200, 136, 64), (130, 2, 2, 72, 200, 64), (500, 3, 4, 264, 72, 128),
+                                               (600, 2, 3, 136, 200, 128), (400, 2, 2, 512, 256, 128)])
 def test_expert_products_over_grouped_rows_and_their_weighted_sum(dtype, T, top, E, H, ff, rows):
     """gate | up with the clamped unit, down, and the sum with identity experts, a shared branch, another branch and a
     bias, against 64-bit products of the same operands; sizes the matrix-core tiles take and sizes they do not (an
