@@ -531,3 +531,28 @@ def test_clamped_gated_unit(dtype):
         got = ops.glu_clamped(gu.to(DEV), 1.5, 1.702).double().cpu()
         want = plain.clamped_unit(gu[:, :I].double(), gu[:, I:].double(), 1.5)
         assert (got - want).abs().max() <= (1e-6 if dtype == torch.float32 else 1e-2) * want.abs().max()
+
+
+@pytest.mark.parametrize("M", [1, 9, 40, 64])
+def test_clamped_gated_unit_on_store_of_the_few_rows_products(M):
+    """gate | up with the clamped unit applied to the 32-bit sums inside the product kernels (the weight-streaming
+    kernel up to 64 rows, the rows kernel up to 128) against 64-bit products of the same operands; with no limit the
+    same kernels still give silu(gate) * up."""
+    from ullm_amd.kernels import ops
+    g = torch.Generator().manual_seed(M)
+    K, I, limit = 256, 192, 1.3
+    x = torch.randn(M, K, generator=g).bfloat16()
+    w = (torch.randn(2 * I, K, generator=g) * 0.15).bfloat16()
+    gu = x.double() @ w.double().T
+    want = plain.clamped_unit(gu[:, :I], gu[:, I:], limit)
+    silu = gu[:, :I] * torch.sigmoid(gu[:, :I]) * gu[:, I:]
+    got = []
+    if M <= 64:
+        got.append((ops.gemm_skinny_silu(x.to(DEV), w.to(DEV), limit=limit, alpha=1.702), want))
+        got.append((ops.gemm_skinny_silu(x.to(DEV), w.to(DEV)), silu))
+    if ops.gemm_rows_supports(x.to(DEV), w.to(DEV), silu=True):
+        got.append((ops.gemm_rows(x.to(DEV), w.to(DEV), silu=True, limit=limit, alpha=1.702), want))
+        got.append((ops.gemm_rows(x.to(DEV), w.to(DEV), silu=True), silu))
+    assert got
+    for out, ref in got:
+        assert (out.double().cpu() - ref).abs().max() <= 1e-2 * ref.abs().max()

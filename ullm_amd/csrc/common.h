@@ -34,6 +34,17 @@ __device__ __forceinline__ float fast_silu(float g) {
   return g * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-1.4426950408889634f * g));
 }
 
+// The gated unit of a feed-forward on the 32-bit sums g (gate half) and u (up half).  limit <= 0: silu(g) * u.
+// Else the clamped unit: g' = min(g, limit), u' = clamp(u, -limit, limit), g' * sigmoid(alpha * g') * (u' + 1).
+__device__ __forceinline__ float gated_unit(float g, float u, float limit, float alpha) {
+  if (limit > 0.f) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return g * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-1.4426950408889634f * alpha * g)) * (u + 1.f);
+  }
+  return fast_silu(g) * u;
+}
+
 __device__ __forceinline__ float ld_f32(const float* p) { return *p; }
 __device__ __forceinline__ float ld_f32(const bf16_t* p) { return bf16_bits_to_f32(*p); }
 __device__ __forceinline__ void st_f32(float* p, float v) { *p = v; }

@@ -63,6 +63,7 @@ struct NormAhead {
 struct RowSquares {
   const float* sq;
   int quads;
+  float unit_limit, unit_alpha;       // EPI_SILU: the gated unit's parameters (limit 0: silu(gate) * up), see gated_unit
 };
 
 
@@ -79,7 +80,7 @@ template <int MT, int NT, int EPI, typename TC, typename RedT>
 __device__ __forceinline__ void skinny_finish(f32x4_t (&acc)[NT][MT], RedT& red, const float* __restrict__ bias,
                                               TC* __restrict__ C, float* __restrict__ R, int ldc, int M, int N, int n0,
                                               bool scaled, const float (*sq)[16 * MT], int K, float eps,
-                                              const NormAhead& ahead) {
+                                              const NormAhead& ahead, float unit_limit = 0.f, float unit_alpha = 0.f) {
   constexpr int OT = EPI == EPI_SILU ? NT / 2 : NT;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
   const int g = lane >> 4, r = lane & 15;
@@ -167,7 +168,8 @@ __device__ __forceinline__ void skinny_finish(f32x4_t (&acc)[NT][MT], RedT& red,
       if (EPI == EPI_SILU) {
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-          if (nn + j < N) st_f32(C + (size_t)m * ldc + nn + j, fast_silu(acc[i][t][j]) * acc[i + OT][t][j]);
+          if (nn + j < N)
+            st_f32(C + (size_t)m * ldc + nn + j, gated_unit(acc[i][t][j], acc[i + OT][t][j], unit_limit, unit_alpha));
       } else if (EPI == EPI_RESADD) {
         float* rp = R + (size_t)m * ldc + nn;
         if (nn + 3 < N) {
@@ -406,7 +408,8 @@ gemm_skinny_kernel(const void* __restrict__ Xv, int ldx, const bf16_t* __restric
   }
   __syncthreads();                                        // the partial sums take the place of the stages
   auto& red = *reinterpret_cast<float (*)[MAXW - 1][NT * MT][64 * 4]>(lds);
-  skinny_finish<MT, NT, EPI, TC>(acc, red, bias, C, R, ldc, M, n_end, n0, scaled, sq, K, eps, ahead);
+  skinny_finish<MT, NT, EPI, TC>(acc, red, bias, C, R, ldc, M, n_end, n0, scaled, sq, K, eps, ahead, before.unit_limit,
+                                 before.unit_alpha);
 }
 
 template <int MT, int NT, int EPI, typename TC, bool NORMX, typename... Args>
@@ -519,7 +522,8 @@ extern "C" int ullm_gemm_skinny_blocks(int M, int N, int K, int ldx, int ldw, in
 }
 
 // X bfloat16 [M, K]; W bfloat16 [N, K] (with epi 2: [2 N, K]).  epi: 0 store to C (c_dtype, bias optional),
-// 1 add into R (float32 [M, N], row stride ldc), 2 silu(gate) * up to C (bfloat16 [M, N]).
+// 1 add into R (float32 [M, N], row stride ldc), 2 silu(gate) * up to C (bfloat16 [M, N]), or with unit_limit > 0
+// the clamped gated unit (gated_unit in common.h) of gate and up.
 // With gain (float32 [K]): X is float32 [M <= 16, K] and its RMS norm with this gain and eps is what
 // is multiplied (epi 0 and 2).  force_nt / force_waves: 0 = chosen here.
 // With next_gain (float32 [N], epi 1): the norm that follows is handed ahead: next_x (bfloat16 [M, N], row stride
@@ -531,7 +535,8 @@ extern "C" int ullm_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
                                 int ldc, int M, int N, int K, int epi, int c_dtype, int force_nt,
                                 int force_waves, const float* gain, float eps, int force_rows,
                                 const float* next_gain, void* next_x, int ld_next, float* next_sq,
-                                const float* row_sq, int sq_parts, hipStream_t stream) {
+                                const float* row_sq, int sq_parts, float unit_limit, float unit_alpha,
+                                hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (!ullm_gemm_skinny_supports(M, N, K, ldx, ldw) || ldc < N) return ULLM_ERR_SHAPE;
   if (((uintptr_t)X & 15) || ((uintptr_t)W & 15)) return ULLM_ERR_SHAPE;
@@ -549,7 +554,8 @@ extern "C" int ullm_gemm_skinny(const void* X, int ldx, const void* W, int ldw, 
   const int mt = plan.mt, nt = plan.nt, rows = plan.rows, tiles = plan.tiles, waves = plan.waves,
             k_per_wave = plan.k_per_wave;
   const NormAhead ahead{next_gain, (bf16_t*)next_x, next_sq, ld_next, (tiles + 3) / 4 * 4};
-  const RowSquares before{row_sq, sq_parts / 4};
+  if (unit_limit > 0.f && epi != EPI_SILU) return ULLM_ERR_UNSUPPORTED;
+  const RowSquares before{row_sq, sq_parts / 4, unit_limit, unit_alpha};
   dim3 grid(tiles), block(64 * waves);
   float* R = (float*)C;
 #define GO_(MT, NT, EPI, TC, NORMX) skinny_launch<MT, NT, EPI, TC, NORMX>(grid, block, stream, X, ldx, \

@@ -566,7 +566,7 @@ def gemm_skinny_supports(a: torch.Tensor, w: torch.Tensor) -> bool:
 
 
 def _gemm_skinny(x, w, bias, c, M, N, K, epi, c_dtype, nt=0, waves=0, gain=None, eps=0.0, rows=0,
-                 ahead=None, squares=None) -> None:
+                 ahead=None, squares=None, unit_limit=0.0, unit_alpha=0.0) -> None:
     """``ahead``: (next gain, next x, next squares) that an adding product leaves for the norm after it;
     ``squares``: the [parts, M] sums such a product left, which scale this product's rows."""
     lib = build.load("gemm_skinny")
@@ -576,7 +576,8 @@ def _gemm_skinny(x, w, bias, c, M, N, K, epi, c_dtype, nt=0, waves=0, gain=None,
                                 _c_int(epi), _c_int(c_dtype), _c_int(nt), _c_int(waves), _p(gain),
                                 ctypes.c_float(eps), _c_int(rows), _p(next_gain), _p(next_x),
                                 _c_int(next_x.stride(0) if next_x is not None else 0), _p(next_sq), _p(squares),
-                                _c_int(squares.shape[1] if squares is not None else 0), _stream()),
+                                _c_int(squares.shape[1] if squares is not None else 0), _c_float(unit_limit),
+                                _c_float(unit_alpha), _stream()),
            "gemm_skinny")
 
 
@@ -640,17 +641,19 @@ def gemm_skinny_add(a: torch.Tensor, w: torch.Tensor, residual: torch.Tensor, nt
 
 
 def gemm_skinny_silu(a: torch.Tensor, w_gate_up: torch.Tensor, nt: int = 0, waves: int = 0, rows: int = 0,
-                     squares: Optional[torch.Tensor] = None, eps: float = 0.0) -> torch.Tensor:
+                     squares: Optional[torch.Tensor] = None, eps: float = 0.0, limit: float = 0.0,
+                     alpha: float = 0.0) -> torch.Tensor:
     """silu(a g^T) * (a u^T) as bfloat16 [M, I] for a (bfloat16 [M, K]) and the stacked weights
     g | u (bfloat16 [2 I, K]); the activation is applied to the 32-bit sums (with ``squares``: to the sums
-    scaled as in :func:`gemm_skinny`)."""
+    scaled as in :func:`gemm_skinny`).  With ``limit`` > 0 the clamped gated unit of :func:`glu_clamped` instead."""
     M, K = a.shape
     two_i, K2 = w_gate_up.shape
     _need(K == K2 and two_i % 2 == 0, f"gate|up weights must be [2 I, {K}]")
     _need(a.dtype == torch.bfloat16 and _skinny_ok(M, K, a, w_gate_up), "gemm_skinny_silu takes bfloat16 [M <= 64, K]")
     out = torch.empty((M, two_i // 2), dtype=torch.bfloat16, device=a.device)
     _check_squares(squares, M)
-    _gemm_skinny(a, w_gate_up, None, out, M, two_i // 2, K, 2, BF16, nt, waves, eps=float(eps), rows=rows, squares=squares)
+    _gemm_skinny(a, w_gate_up, None, out, M, two_i // 2, K, 2, BF16, nt, waves, eps=float(eps), rows=rows, squares=squares,
+                 unit_limit=float(limit), unit_alpha=float(alpha))
     return out
 
 
@@ -728,12 +731,14 @@ def gemm_rows_supports(a: torch.Tensor, w: torch.Tensor, silu: bool = False) -> 
 
 
 def gemm_rows(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, silu: bool = False,
-              squares: Optional[torch.Tensor] = None, eps: float = 0.0) -> torch.Tensor:
+              squares: Optional[torch.Tensor] = None, eps: float = 0.0, limit: float = 0.0,
+              alpha: float = 0.0) -> torch.Tensor:
     """a (bfloat16 [M <= 128, K]) times w (bfloat16 [N, K]) transposed (+ bias float32 [N]) as bfloat16 [M, N];
     with ``silu``, w is gate | up [2 I, K] and the result silu(gate) * up [M, I] on the 32-bit sums.  The
     matrix is cut into one block per compute unit and every wave keeps several stages of its rows of w in
     flight: for the row counts between the few-rows kernel and the library.  ``squares``, ``eps``: as in
-    :func:`gemm_skinny`."""
+    :func:`gemm_skinny`.  With ``silu`` and ``limit`` > 0 the clamped gated unit of :func:`glu_clamped` instead."""
+    _need(silu or limit <= 0, "the clamped unit needs gate | up weights")
     M, K = a.shape
     _need(gemm_rows_supports(a, w, silu), "gemm_rows takes bfloat16, M <= 128, K a multiple of 64, N a multiple of 4")
     n_out = w.shape[0] // 2 if silu else w.shape[0]
@@ -746,7 +751,8 @@ def gemm_rows(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = N
                                                   _c_int(n_out), _c_int(M), _c_int(n_out), _c_int(K),
                                                   _c_int(1 if silu else 0), _p(squares),
                                                   _c_int(squares.shape[1] if squares is not None else 0),
-                                                  ctypes.c_float(float(eps)), _stream()), "gemm_rows")
+                                                  ctypes.c_float(float(eps)), _c_float(float(limit)), _c_float(float(alpha)),
+                                                  _stream()), "gemm_rows")
     return out
 
 

@@ -80,17 +80,21 @@ def add_into_stream(x: torch.Tensor, weight: torch.Tensor, residual: torch.Tenso
     return None
 
 
-def gate_up(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+def gate_up(x: torch.Tensor, weight: torch.Tensor, limit: float = 0.0, alpha: float = 0.0) -> torch.Tensor:
     """silu(x g^T) * (x u^T) for the stacked weights g | u [2 I, K]: by the few-rows kernel or the kernel for up
     to 128 rows with the activation on store, up to the row counts the matrix's limits name; else by the
-    library product and the activation kernel (float32 always: the 32-bit product, then the kernel)."""
+    library product and the activation kernel (float32 always: the 32-bit product, then the kernel).  With
+    ``limit`` > 0 the clamped gated unit (``ops.glu_clamped``) in place of silu(gate) * up, by the same kernels."""
     rows = x.shape[0]
     if x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16:
         lim = dispatch.limits(weight.shape[0], weight.shape[1])
+        unit = dict(limit=limit, alpha=alpha) if limit > 0 else {}
         if rows <= lim.silu_skinny and ops.gemm_skinny_supports(x, weight):
-            return ops.gemm_skinny_silu(x, weight)
+            return ops.gemm_skinny_silu(x, weight, **unit)
         if rows <= min(lim.silu_rows, ops.ROWS_MAX_ROWS) and ops.gemm_rows_supports(x, weight, silu=True):
-            return ops.gemm_rows(x, weight, silu=True)
+            return ops.gemm_rows(x, weight, silu=True, **unit)
+    if limit > 0:
+        return ops.glu_clamped(linear(x, weight), limit, alpha)
     return ops.silu_mul(linear(x, weight))
 
 

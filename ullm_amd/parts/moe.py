@@ -23,7 +23,7 @@ import torch
 
 from ..kernels import ops
 from .base import FeedForward, PartEnv, StepContext, WeightDecl, register_part
-from .linear import linear
+from .linear import gate_up, linear
 
 DEFAULT_NAMES = {"router": "router", "correction": "correction", "expert": "e{index}", "gate": "gate", "up": "up",
                  "down": "down", "shared": "shared"}
@@ -120,6 +120,7 @@ class RoutedExperts(FeedForward):
             y = ops.moe_rows(act, None, self.w_down, tiles, tile_rows, T * self.top, gated=False)
         shared = None
         if self.shared_ff:
-            act = ops.glu_clamped(linear(x, self.w_shared_gate_up), self.shared_limit, self.alpha)
+            # gate | up with the unit on store where the few-rows kernels take the step, as the dense feed-forward's
+            act = gate_up(x, self.w_shared_gate_up, self.shared_limit, self.alpha)
             shared = linear(act, self.w_shared_down)
         return ops.moe_combine(y, x, ids, weights, slot_of_pair, self.experts, base=base, bias=bias, shared=shared)
